@@ -1,0 +1,150 @@
+/*
+ * vtl_hip.h - C ABI of libvtlhip.so, the MI355X (gfx950) backend of VTL's
+ * INT8 quantized-linear path.
+ *
+ * The reference is a V library; V binds C with `fn C.name(...) int` plus
+ * `#flag -lvtlhip` / `#include "vtl_hip.h"`.  Every entry point below is what
+ * one of the reference's V call sites would bind; the site it replaces or
+ * mirrors is cited (paths relative to the reference tree).
+ *
+ * Conventions (taken from the reference's CUDA call sites,
+ * storage/cuda_d_cuda.v:39-42,74-77):
+ *   - every function returns an int status, 0 = success; the V side turns a
+ *     non-zero status into `error(...)` and the layer falls back to its CPU
+ *     path (nn/layers/linear_forward_f32.v:8-11);
+ *   - no exceptions, no aborts: null pointers, negative or mismatching sizes
+ *     return VTL_HIP_ERR_INVALID_ARG;
+ *   - all pointers given to compute entry points are DEVICE pointers obtained
+ *     from vtl_hip_malloc (the owner is the V-side HipStorage, released
+ *     explicitly as in storage/cuda_d_cuda.v:98-102); host memory is touched
+ *     only by the memcpy calls, which block until the copy is done;
+ *   - compute entry points enqueue on the library's current stream (the null
+ *     stream unless vtl_hip_set_stream was called) and return without
+ *     waiting; a later blocking memcpy or vtl_hip_sync orders after them;
+ *   - matrices are dense row-major; weights are passed AS STORED by
+ *     LinearLayer, `[out_features, in_features]` (nn/layers/linear.v:10-16),
+ *     never as a transposed view;
+ *   - one host thread per device; the library keeps no pointers to caller
+ *     memory after a call returns.
+ */
+#ifndef VTL_HIP_H
+#define VTL_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    VTL_HIP_OK = 0,
+    VTL_HIP_ERR_INVALID_ARG = 1, /* null pointer, bad size, bad flag */
+    VTL_HIP_ERR_NO_DEVICE = 2,   /* no usable GPU / bad device id */
+    VTL_HIP_ERR_RUNTIME = 3,     /* a HIP runtime call failed */
+    VTL_HIP_ERR_OUT_OF_MEMORY = 4,
+    VTL_HIP_ERR_UNSUPPORTED = 5  /* shape outside what the kernels cover */
+};
+
+/* ---- device, memory, transfer ------------------------------------------ */
+
+/* cuda.get_device(id) in storage/cuda_d_cuda.v:33. */
+int vtl_hip_device_count(int *n);
+int vtl_hip_set_device(int device_id);
+/* Name and compute-unit count of the current device (diagnostics only). */
+int vtl_hip_device_info(char *name, size_t name_cap, int *compute_units, int *clock_mhz);
+
+/* C.cudaMalloc storage/cuda_d_cuda.v:39; C.cudaFree :100. */
+int vtl_hip_malloc(void **dptr, size_t bytes);
+int vtl_hip_free(void *dptr);
+
+/* C.cudaMemcpy H2D storage/cuda_d_cuda.v:46, D2H :74,:90 (blocking). */
+int vtl_hip_memcpy_h2d(void *dst_device, const void *src_host, size_t bytes);
+int vtl_hip_memcpy_d2h(void *dst_host, const void *src_device, size_t bytes);
+int vtl_hip_memcpy_d2d(void *dst_device, const void *src_device, size_t bytes);
+int vtl_hip_memset(void *dst_device, int byte_value, size_t bytes);
+
+/* Wait for everything enqueued on the current stream. */
+int vtl_hip_sync(void);
+
+/* Stream the compute entry points enqueue on (a hipStream_t, NULL = null
+ * stream).  The reference has no stream concept beyond the unused field at
+ * storage/cuda_notd_cuda.v:9. */
+int vtl_hip_set_stream(void *hip_stream);
+int vtl_hip_get_stream(void **hip_stream);
+
+/* Timing helpers (hipEvent on the current stream); the reference times with
+ * wall-clock ticks, benchmarks/vs_numpy/matmul_bench.v:41-43. */
+int vtl_hip_event_create(void **event);
+int vtl_hip_event_destroy(void *event);
+int vtl_hip_event_record(void *event);
+int vtl_hip_event_elapsed_ms(void *start, void *stop, float *ms);
+
+/* ---- quantization vocabulary -------------------------------------------- */
+
+/* absmax_out[0] = max |x| over the tensor (per_row == 0) or absmax_out[r] =
+ * max |x[r, :]| (per_row != 0).  NaN elements are ignored; empty -> 0.
+ * Replaces Tensor.abs (math.v:11-16) + max_axis (reduction.v:163-232) /
+ * stats.max (stats/stats.v:401-407). */
+int vtl_hip_absmax_f32(const float *x, int64_t rows, int64_t cols, int per_row,
+                       float *absmax_out);
+
+/* scale = absmax / 127 (f32 division); q = clamp(round_half_even(x / scale),
+ * -127, 127) with NaN -> 0 and scale 0 -> all codes 0.  scale_out receives 1
+ * (per_row == 0) or `rows` scales.  Replaces divide_scalar (math_op.v:103-111)
+ * + round_to_even (math.v:570-574) + clamp (autograd/variable_ops.v:228-248)
+ * + as_i8 (cast.v:107-121). */
+int vtl_hip_quantize_f32_i8(const float *x, int64_t rows, int64_t cols, int per_row,
+                            int8_t *q, float *scale_out);
+
+/* Same codes, but with scales the caller already holds on the device. */
+int vtl_hip_quantize_with_scale_f32_i8(const float *x, const float *scale, int64_t rows,
+                                       int64_t cols, int per_row, int8_t *q);
+
+/* x[r,c] = f32(q[r,c]) * scale[r or 0].  Replaces as_f32 (cast.v:35) +
+ * multiply_scalar (math_op.v:137-145). */
+int vtl_hip_dequantize_i8_f32(const int8_t *q, const float *scale, int64_t rows, int64_t cols,
+                              int per_row, float *x);
+
+/* ---- matmul -------------------------------------------------------------- */
+
+/* C[M,N] (i32) = A[M,K] (i8) . Bt[N,K]^T (i8), exact.  The int8 counterpart
+ * of la.matmul (la/la.v:38-55) / gate_matmul (autograd/gates_blas.v:6-23) /
+ * gemm_cuda (tensor_cuda_d_cuda.v:155-177) with the second operand given
+ * K-contiguous.  K <= 131072 so that |acc| <= K * 127^2 < 2^31. */
+int vtl_hip_gemm_i8_i32(const int8_t *A, const int8_t *Bt, int32_t *C, int M, int N, int K);
+
+/* Y[m,n] = fl(fl(f32(acc) * fl(sa[m] * sw[n])) + bias[n]), ReLU if relu != 0
+ * (x < 0 -> 0, nn/internal/activation.v:63-70).  sa: M scales when
+ * sa_per_row else 1; sw: N scales when sw_per_col else 1; bias: N floats or
+ * NULL (no addition).  The int8 form of linear_forward_f32
+ * (nn/layers/linear_forward_f32.v:7-18): y = x.W^T + b with W as stored. */
+int vtl_hip_linear_i8_f32(const int8_t *A, const float *sa, int sa_per_row,
+                          const int8_t *Wq, const float *sw, int sw_per_col,
+                          const float *bias, float *Y, int M, int N, int K, int relu);
+
+/* Per-token (row) quantization of X[M,K] on the fly, then the int8 linear
+ * against per-output-channel quantized weights.  workspace: device scratch
+ * of at least vtl_hip_linear_f32_dynquant_workspace(M, K) bytes, owned by
+ * the caller (the reference's DeviceSession keeps such staging buffers,
+ * autograd_cuda/device_session.v:13-24). */
+size_t vtl_hip_linear_f32_dynquant_workspace(int M, int K);
+int vtl_hip_linear_f32_dynquant(const float *X, const int8_t *Wq, const float *sw,
+                                const float *bias, float *Y, int M, int N, int K, int relu,
+                                void *workspace, size_t workspace_bytes);
+
+/* ReLU in place on the device (nn/internal/activation.v:63-70,
+ * relu_cuda tensor_cuda_d_cuda.v:205-235). */
+int vtl_hip_relu_f32(float *x, int64_t n);
+
+/* ---- diagnostics ---------------------------------------------------------- */
+
+const char *vtl_hip_strerror(int status);
+/* Text of the last HIP runtime error seen by this thread ("" if none). */
+const char *vtl_hip_last_error(void);
+const char *vtl_hip_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

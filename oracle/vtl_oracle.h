@@ -1,0 +1,112 @@
+/*
+ * vtl_oracle.h - CPU restatement of the INT8 quantized-linear arithmetic that
+ * sits behind vtl.Tensor[T] / Sequential.linear().
+ *
+ * THIS IS TEST INFRASTRUCTURE, NOT PRODUCT CODE.  Only the test-suite, the
+ * smoke check and the CPU-baseline leg of the benchmark may link or load it.
+ * The product library (libvtlhip.so) never calls into it and has no CPU
+ * fallback of its own.
+ *
+ * The reference (a pure-V library) has no composed INT8 path; the contract
+ * below is composed from the reference's CPU vocabulary, cited per function.
+ * All paths are relative to the reference tree.
+ *
+ * Spec decisions that the reference cannot settle (none of its tests reach
+ * them) and that this oracle fixes:
+ *   - NaN elements are ignored by absmax (max_axis's `val > best` compare,
+ *     reduction.v:198-203, never selects a NaN that is not first); an
+ *     all-NaN or empty slice has absmax 0.
+ *   - absmax == 0  -> scale 0, every code 0, dequantized 0.
+ *   - NaN quotient -> code 0 (what an x86 float->int cast followed by the
+ *     narrowing to i8 yields on the reference's CPU path).
+ *   - +-Inf input  -> absmax Inf, scale Inf, finite x -> 0, +-Inf -> NaN -> 0.
+ *   - -128 is never produced.
+ *
+ * Pinning status (which independent check pins each function) is listed in
+ * the header of vtl_oracle.c.
+ */
+#ifndef VTL_ORACLE_H
+#define VTL_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* absmax over the whole tensor (per_row == 0, out[1]) or per row
+ * (per_row != 0, out[rows]).  abs: math.v:11-16; max: math.v:468-472,
+ * max_axis: reduction.v:163-232, stats.max: stats/stats.v:401-407. */
+void vtl_ref_absmax_f32(const float *x, int64_t rows, int64_t cols, int per_row, float *out);
+
+/* scale = absmax / 127 in f32 (divide_scalar in T: math_op.v:103-111). */
+float vtl_ref_scale_from_absmax(float absmax);
+
+/* One code: clamp(round_half_even(x / scale), -127, 127).
+ * divide_scalar math_op.v:103-111, round_to_even math.v:570-574,
+ * clamp autograd/variable_ops.v:228-248. */
+int8_t vtl_ref_quantize_one(float x, float scale);
+
+/* Symmetric quantize: computes scales (1 or rows of them) and codes. */
+void vtl_ref_quantize_f32_i8(const float *x, int64_t rows, int64_t cols, int per_row,
+                             int8_t *q, float *scale_out);
+
+/* Quantize with caller-supplied scales (1 or rows of them). */
+void vtl_ref_quantize_with_scale(const float *x, const float *scale, int64_t rows, int64_t cols,
+                                 int per_row, int8_t *q);
+
+/* x_hat = f32(q) * scale (multiply_scalar math_op.v:137-145). */
+void vtl_ref_dequantize_i8_f32(const int8_t *q, const float *scale, int64_t rows, int64_t cols,
+                               int per_row, float *x);
+
+/* C[M,N] (i32) = A[M,K] (i8, row-major) . Bt[N,K]^T (i8, row-major: the
+ * weight as LinearLayer stores it, nn/layers/linear.v:10-16).  Shape rule
+ * of la.matmul la/la.v:38-43.  threads <= 1: single thread (the reference is
+ * single-threaded); otherwise OpenMP over rows. */
+void vtl_ref_gemm_i8_i32(const int8_t *A, const int8_t *Bt, int32_t *C,
+                         int64_t M, int64_t N, int64_t K, int threads);
+
+/* Y[m,n] = fl(fl(fl((float)acc) * fl(sa[m]*sw[n])) + bias[n]), then optional
+ * ReLU (x < 0 -> 0, nn/internal/activation.v:63-70).  sa has M entries when
+ * sa_per_row else 1; sw has N entries when sw_per_col else 1; bias may be
+ * NULL (no add at all).  Bias broadcast [1,N] over [M,N]: math_op.v:9-21. */
+void vtl_ref_epilogue_f32(const int32_t *acc, const float *sa, int sa_per_row,
+                          const float *sw, int sw_per_col, const float *bias,
+                          float *Y, int64_t M, int64_t N, int relu);
+
+/* gemm + epilogue in one call. */
+void vtl_ref_linear_i8_f32(const int8_t *A, const float *sa, int sa_per_row,
+                           const int8_t *Wq, const float *sw, int sw_per_col,
+                           const float *bias, float *Y,
+                           int64_t M, int64_t N, int64_t K, int relu, int threads);
+
+/* Per-token dynamic quantization of X[M,K] followed by the int8 linear. */
+void vtl_ref_linear_f32_dynquant(const float *X, const int8_t *Wq, const float *sw,
+                                 const float *bias, float *Y,
+                                 int64_t M, int64_t N, int64_t K, int relu, int threads);
+
+/* ReLU in place (nn/internal/activation.v:63-70). */
+void vtl_ref_relu_f32(float *x, int64_t n);
+
+/* The reference's existing f32 Linear as documented: y = x.W^T + b through
+ * f64 (la/la.v:44-53: as_f64 -> f64 GEMM -> as_f32; then Tensor.add,
+ * nn/layers/linear_forward_f32.v:16-18), with the explicit transpose the
+ * reference's own device session uses (autograd_cuda/device_session.v:38-46).
+ * The f64 summation order inside the un-vendored VSL GEMM is unknown, so
+ * values are pinned only up to f64 rounding: parity unpinned beyond that. */
+void vtl_ref_linear_f32_via_f64(const float *X, const float *W, const float *bias, float *Y,
+                                int64_t M, int64_t N, int64_t K);
+
+/* Row-parallel forms (same arithmetic), for timing the CPU baseline on all cores. */
+void vtl_ref_quantize_f32_i8_mt(const float *x, int64_t rows, int64_t cols, int per_row,
+                                int8_t *q, float *scale_out, int threads);
+void vtl_ref_dequantize_i8_f32_mt(const int8_t *q, const float *scale, int64_t rows, int64_t cols,
+                                  int per_row, float *x, int threads);
+
+int vtl_ref_max_threads(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

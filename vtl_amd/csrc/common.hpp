@@ -1,0 +1,30 @@
+// Shared declarations of libvtlhip.so (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "vtl_hip.h"
+
+namespace vtlhip {
+
+// Stream every compute entry point enqueues on (nullptr = the null stream).
+hipStream_t current_stream();
+
+// Records a failed HIP runtime call for vtl_hip_last_error() and maps it to a
+// status code of the C ABI.
+int record_hip_error(hipError_t e, const char *what);
+
+// Checks the launch that was just made.
+int check_launch(const char *kernel_name);
+
+constexpr int kWave = 64;
+
+}  // namespace vtlhip
+
+#define VTL_HIP_TRY(expr)                                                  \
+    do {                                                                   \
+        hipError_t vtl_e_ = (expr);                                        \
+        if (vtl_e_ != hipSuccess)                                          \
+            return ::vtlhip::record_hip_error(vtl_e_, #expr);              \
+    } while (0)

@@ -1,0 +1,598 @@
+// Symmetric INT8 quantization vocabulary for gfx950: absmax, quantize,
+// dequantize, ReLU.  All of it is HBM-bound streaming work: 16-byte loads per
+// lane, coalesced across the 64-wide wavefront, one pass over the data where
+// the row fits in registers, wavefront reductions through cross-lane moves and
+// one LDS exchange per workgroup.
+//
+// Arithmetic contract (per element, f32):
+//   absmax = max |x|            NaN ignored (v_max_f32 returns the non-NaN)
+//   scale  = absmax / 127       IEEE division, correctly rounded
+//   code   = clamp(rne(x / scale), -127, 127), NaN -> 0
+//   x_hat  = f32(code) * scale
+// The division is the correctly rounded one.  The quotient is first estimated
+// with x * (1/scale); only when that estimate is too close to a rounding tie
+// to decide the integer is the exact division evaluated (see quant_code).
+#include "common.hpp"
+
+using namespace vtlhip;
+
+namespace {
+
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef int int4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float wave_max(float v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1)
+        v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+// Max over the workgroup; every thread gets the result.  smem holds T/64
+// floats and is used once per kernel.
+template <int T>
+__device__ __forceinline__ float block_max(float v, float *smem)
+{
+    v = wave_max(v);
+    if constexpr (T > 64) {
+        const int w = threadIdx.x >> 6;
+        if ((threadIdx.x & 63) == 0)
+            smem[w] = v;
+        __syncthreads();
+        float r = smem[0];
+#pragma unroll
+        for (int i = 1; i < T / 64; i++)
+            r = fmaxf(r, smem[i]);
+        v = r;
+    }
+    return v;
+}
+
+__device__ __forceinline__ float absmax4(float m, float4_t v)
+{
+    m = fmaxf(m, fabsf(v.x));
+    m = fmaxf(m, fabsf(v.y));
+    m = fmaxf(m, fabsf(v.z));
+    m = fmaxf(m, fabsf(v.w));
+    return m;
+}
+
+// Saturating f32 -> i32 conversion; NaN converts to 0 in hardware.
+__device__ __forceinline__ int cvt_i32_sat(float r)
+{
+    int i;
+    asm("v_cvt_i32_f32 %0, %1" : "=v"(i) : "v"(r));
+    return i;
+}
+
+struct QuantScale {
+    float scale;
+    float rinv;  // 1/scale when `fast`
+    bool fast;   // scale and 1/scale are normal numbers with headroom
+};
+
+__device__ __forceinline__ QuantScale make_quant_scale(float scale)
+{
+    QuantScale p;
+    p.scale = scale;
+    p.fast = (scale >= 0x1p-100f) && (scale <= 0x1p100f);
+    p.rinv = p.fast ? (1.0f / scale) : 0.0f;
+    return p;
+}
+
+// Half-width of the band around k + 0.5 inside which the estimated quotient
+// cannot decide the rounding.  For |x/scale| <= 128 the estimate
+// fl(x * fl(1/scale)) is within 2^-16 of the true quotient and the correctly
+// rounded quotient within 2^-18, so 2^-14 leaves a factor of three.  Larger
+// quotients clamp to +-127 whichever way they round.
+constexpr float kTieBand = 0x1p-14f;
+
+__device__ __forceinline__ int quant_code(float x, const QuantScale &p)
+{
+    float r;
+    if (p.fast) {
+        const float t = x * p.rinv;
+        r = rintf(t);
+        if (__builtin_expect(fabsf(t - r) >= 0.5f - kTieBand, 0))
+            r = rintf(x / p.scale);
+    } else {
+        r = rintf(x / p.scale);  // 0/0, x/Inf, subnormal scales: exact path
+    }
+    const int i = cvt_i32_sat(r);
+    return min(max(i, -127), 127);
+}
+
+__device__ __forceinline__ unsigned pack4(int a, int b, int c, int d)
+{
+    return (unsigned)(a & 0xff) | ((unsigned)(b & 0xff) << 8) | ((unsigned)(c & 0xff) << 16) |
+           ((unsigned)d << 24);
+}
+
+__device__ __forceinline__ unsigned quant4(float4_t v, const QuantScale &p)
+{
+    return pack4(quant_code(v.x, p), quant_code(v.y, p), quant_code(v.z, p), quant_code(v.w, p));
+}
+
+// ---- absmax ----------------------------------------------------------------
+
+// One workgroup per row, strided loop over the row.
+template <int T, int VEC>
+__global__ __launch_bounds__(T) void absmax_rows_kernel(const float *__restrict__ x, int64_t cols,
+                                                        float *__restrict__ out)
+{
+    __shared__ float smem[T / 64];
+    const int64_t row = blockIdx.x;
+    const float *xr = x + row * cols;
+    float m = 0.0f;
+    if constexpr (VEC == 4) {
+        const float4_t *xv = reinterpret_cast<const float4_t *>(xr);
+        const int64_t nv = cols >> 2;
+        for (int64_t i = threadIdx.x; i < nv; i += T)
+            m = absmax4(m, xv[i]);
+    } else {
+        for (int64_t i = threadIdx.x; i < cols; i += T)
+            m = fmaxf(m, fabsf(xr[i]));
+    }
+    m = block_max<T>(m, smem);
+    if (threadIdx.x == 0)
+        out[row] = m;
+}
+
+// Whole-tensor absmax: grid-stride pass, one atomic max per workgroup on the
+// bit pattern (non-negative floats order like unsigned integers).
+template <int T>
+__global__ __launch_bounds__(T) void absmax_flat_kernel(const float *__restrict__ x, int64_t n,
+                                                        int vec_ok, unsigned *__restrict__ out_bits)
+{
+    __shared__ float smem[T / 64];
+    float m = 0.0f;
+    const int64_t tid = (int64_t)blockIdx.x * T + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * T;
+    if (vec_ok) {
+        const float4_t *xv = reinterpret_cast<const float4_t *>(x);
+        const int64_t nv = n >> 2;
+        for (int64_t i = tid; i < nv; i += stride)
+            m = absmax4(m, xv[i]);
+        if (tid < (n & 3))
+            m = fmaxf(m, fabsf(x[(nv << 2) + tid]));
+    } else {
+        for (int64_t i = tid; i < n; i += stride)
+            m = fmaxf(m, fabsf(x[i]));
+    }
+    m = block_max<T>(m, smem);
+    if (threadIdx.x == 0)
+        atomicMax(out_bits, __float_as_uint(m));
+}
+
+__global__ void fill_u32_kernel(unsigned *p, unsigned v, int64_t n)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n)
+        p[i] = v;
+}
+
+__global__ void scale_from_absmax_kernel(float *inout, int64_t n)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n)
+        inout[i] = inout[i] / 127.0f;
+}
+
+// ---- fused per-row absmax + quantize ---------------------------------------
+
+// One workgroup per row; the row stays in registers between the absmax pass
+// and the quantize pass, so HBM sees 4 bytes in and 1 byte out per element.
+// Requires cols % 4 == 0 and cols <= 4 * T * NV.
+template <int T, int NV>
+__global__ __launch_bounds__(T) void quantize_rows_reg_kernel(const float *__restrict__ x,
+                                                              int64_t cols, int8_t *__restrict__ q,
+                                                              float *__restrict__ scale_out)
+{
+    __shared__ float smem[T / 64];
+    const int64_t row = blockIdx.x;
+    const float4_t *xv = reinterpret_cast<const float4_t *>(x + row * cols);
+    unsigned *qv = reinterpret_cast<unsigned *>(q + row * cols);
+    const int nv = (int)(cols >> 2);
+
+    float4_t v[NV];
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int idx = i * T + threadIdx.x;
+        if (idx < nv)
+            v[i] = __builtin_nontemporal_load(xv + idx);
+        else
+            v[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+    }
+    float m = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NV; i++)
+        m = absmax4(m, v[i]);
+    m = block_max<T>(m, smem);
+
+    const float scale = m / 127.0f;
+    if (threadIdx.x == 0)
+        scale_out[row] = scale;
+    const QuantScale p = make_quant_scale(scale);
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int idx = i * T + threadIdx.x;
+        if (idx < nv)
+            __builtin_nontemporal_store(quant4(v[i], p), qv + idx);
+    }
+}
+
+// Rows too long for registers, or not a multiple of four: two passes over the
+// row inside one workgroup (the second pass mostly hits L2 / MALL).
+template <int T, int VEC>
+__global__ __launch_bounds__(T) void quantize_rows_loop_kernel(const float *__restrict__ x,
+                                                               int64_t cols, int8_t *__restrict__ q,
+                                                               float *__restrict__ scale_out)
+{
+    __shared__ float smem[T / 64];
+    const int64_t row = blockIdx.x;
+    const float *xr = x + row * cols;
+    int8_t *qr = q + row * cols;
+    float m = 0.0f;
+    if constexpr (VEC == 4) {
+        const float4_t *xv = reinterpret_cast<const float4_t *>(xr);
+        const int64_t nv = cols >> 2;
+        for (int64_t i = threadIdx.x; i < nv; i += T)
+            m = absmax4(m, xv[i]);
+    } else {
+        for (int64_t i = threadIdx.x; i < cols; i += T)
+            m = fmaxf(m, fabsf(xr[i]));
+    }
+    m = block_max<T>(m, smem);
+    const float scale = m / 127.0f;
+    if (threadIdx.x == 0)
+        scale_out[row] = scale;
+    const QuantScale p = make_quant_scale(scale);
+    if constexpr (VEC == 4) {
+        const float4_t *xv = reinterpret_cast<const float4_t *>(xr);
+        unsigned *qv = reinterpret_cast<unsigned *>(qr);
+        const int64_t nv = cols >> 2;
+        for (int64_t i = threadIdx.x; i < nv; i += T)
+            qv[i] = quant4(xv[i], p);
+    } else {
+        for (int64_t i = threadIdx.x; i < cols; i += T)
+            qr[i] = (int8_t)quant_code(xr[i], p);
+    }
+}
+
+// ---- quantize with scales already on the device ----------------------------
+
+// per_row: block (x = row, y = chunk of the row); flat: block x = chunk of the
+// whole tensor.  A chunk is 4 * T * NV elements (VEC == 4) or T * NV (VEC == 1).
+template <int T, int NV, int VEC>
+__global__ __launch_bounds__(T) void quantize_scaled_kernel(const float *__restrict__ x,
+                                                            const float *__restrict__ scale,
+                                                            int per_row, int64_t cols,
+                                                            int8_t *__restrict__ q)
+{
+    const int64_t row = per_row ? (int64_t)blockIdx.x : 0;
+    const int64_t chunk = per_row ? (int64_t)blockIdx.y : (int64_t)blockIdx.x;
+    const float *xr = x + row * cols;
+    int8_t *qr = q + row * cols;
+    const QuantScale p = make_quant_scale(scale[row]);
+    if constexpr (VEC == 4) {
+        const float4_t *xv = reinterpret_cast<const float4_t *>(xr);
+        unsigned *qv = reinterpret_cast<unsigned *>(qr);
+        const int64_t nv = cols >> 2;
+        const int64_t base = chunk * (T * NV);
+        float4_t v[NV];
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            const int64_t idx = base + i * T + threadIdx.x;
+            if (idx < nv)
+                v[i] = __builtin_nontemporal_load(xv + idx);
+        }
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            const int64_t idx = base + i * T + threadIdx.x;
+            if (idx < nv)
+                __builtin_nontemporal_store(quant4(v[i], p), qv + idx);
+        }
+        // ragged tail of a flat tensor (cols % 4 elements)
+        if (chunk == 0 && threadIdx.x < (cols & 3)) {
+            const int64_t idx = (nv << 2) + threadIdx.x;
+            qr[idx] = (int8_t)quant_code(xr[idx], p);
+        }
+    } else {
+        const int64_t base = chunk * (T * NV);
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            const int64_t idx = base + i * T + threadIdx.x;
+            if (idx < cols)
+                qr[idx] = (int8_t)quant_code(xr[idx], p);
+        }
+    }
+}
+
+// ---- dequantize -------------------------------------------------------------
+
+// Same block indexing as quantize_scaled_kernel.  Each lane reads four codes
+// (4 bytes) and writes one 16-byte vector, so both sides stay coalesced.
+template <int T, int NV, int VEC>
+__global__ __launch_bounds__(T) void dequantize_kernel(const int8_t *__restrict__ q,
+                                                       const float *__restrict__ scale, int per_row,
+                                                       int64_t cols, float *__restrict__ x)
+{
+    const int64_t row = per_row ? (int64_t)blockIdx.x : 0;
+    const int64_t chunk = per_row ? (int64_t)blockIdx.y : (int64_t)blockIdx.x;
+    const int8_t *qr = q + row * cols;
+    float *xr = x + row * cols;
+    const float s = scale[row];
+    if constexpr (VEC == 4) {
+        const unsigned *qv = reinterpret_cast<const unsigned *>(qr);
+        float4_t *xv = reinterpret_cast<float4_t *>(xr);
+        const int64_t nv = cols >> 2;
+        const int64_t base = chunk * (T * NV);
+        unsigned c[NV];
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            const int64_t idx = base + i * T + threadIdx.x;
+            c[i] = (idx < nv) ? __builtin_nontemporal_load(qv + idx) : 0u;
+        }
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            const int64_t idx = base + i * T + threadIdx.x;
+            if (idx < nv) {
+                const int w = (int)c[i];
+                float4_t o;
+                o.x = (float)((w << 24) >> 24) * s;
+                o.y = (float)((w << 16) >> 24) * s;
+                o.z = (float)((w << 8) >> 24) * s;
+                o.w = (float)(w >> 24) * s;
+                __builtin_nontemporal_store(o, xv + idx);
+            }
+        }
+        if (chunk == 0 && threadIdx.x < (cols & 3)) {
+            const int64_t idx = (nv << 2) + threadIdx.x;
+            xr[idx] = (float)qr[idx] * s;
+        }
+    } else {
+        const int64_t base = chunk * (T * NV);
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            const int64_t idx = base + i * T + threadIdx.x;
+            if (idx < cols)
+                xr[idx] = (float)qr[idx] * s;
+        }
+    }
+}
+
+// ---- ReLU --------------------------------------------------------------------
+
+__global__ __launch_bounds__(256) void relu_kernel(float *__restrict__ x, int64_t n)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) {
+        const float v = x[i];
+        if (v < 0.0f)  // NaN and -0.0 pass through, as on the CPU path
+            x[i] = 0.0f;
+    }
+}
+
+inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+constexpr int64_t kMaxGridX = 2147483647LL;
+constexpr int64_t kMaxGridY = 65535;
+
+int check_2d(const void *a, const void *b, int64_t rows, int64_t cols)
+{
+    if (!a || !b || rows < 0 || cols < 0)
+        return VTL_HIP_ERR_INVALID_ARG;
+    if (rows > kMaxGridX)
+        return VTL_HIP_ERR_UNSUPPORTED;
+    if (cols > 0 && rows > INT64_MAX / cols)
+        return VTL_HIP_ERR_INVALID_ARG;
+    return VTL_HIP_OK;
+}
+
+int launch_fill_zero(float *p, int64_t n, hipStream_t st)
+{
+    const int64_t blocks = (n + 255) / 256;
+    hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)blocks), dim3(256), 0, st,
+                       reinterpret_cast<unsigned *>(p), 0u, n);
+    return check_launch("fill_u32_kernel");
+}
+
+}  // namespace
+
+namespace vtlhip {
+
+// Per-row fused quantize; used by the C entry point and by the dynamic-quant
+// linear.  Preconditions were checked by the caller.
+int launch_quantize_rows(const float *x, int64_t rows, int64_t cols, int8_t *q, float *scale_out,
+                         hipStream_t st)
+{
+    if (rows == 0)
+        return VTL_HIP_OK;
+    if (cols == 0)
+        return launch_fill_zero(scale_out, rows, st);
+    const bool vec = (cols % 4 == 0) && aligned(x, 16) && aligned(q, 4);
+    const dim3 grid((unsigned)rows);
+#define VTL_Q_REG(T, NV)                                                                    \
+    hipLaunchKernelGGL((quantize_rows_reg_kernel<T, NV>), grid, dim3(T), 0, st, x, cols, q, \
+                       scale_out)
+    if (vec && cols <= 4 * 64 * 1)
+        VTL_Q_REG(64, 1);
+    else if (vec && cols <= 4 * 64 * 4)
+        VTL_Q_REG(64, 4);
+    else if (vec && cols <= 4 * 256 * 4)
+        VTL_Q_REG(256, 4);
+    else if (vec && cols <= 4 * 256 * 16)
+        VTL_Q_REG(256, 16);
+    else if (vec && cols <= 4 * 1024 * 16)
+        VTL_Q_REG(1024, 16);
+    else if (vec)
+        hipLaunchKernelGGL((quantize_rows_loop_kernel<1024, 4>), grid, dim3(1024), 0, st, x, cols, q,
+                           scale_out);
+    else
+        hipLaunchKernelGGL((quantize_rows_loop_kernel<256, 1>), grid, dim3(256), 0, st, x, cols, q,
+                           scale_out);
+#undef VTL_Q_REG
+    return check_launch("quantize_rows");
+}
+
+}  // namespace vtlhip
+
+extern "C" {
+
+int vtl_hip_absmax_f32(const float *x, int64_t rows, int64_t cols, int per_row, float *absmax_out)
+{
+    int st = check_2d(x, absmax_out, rows, cols);
+    if (st != VTL_HIP_OK)
+        return st;
+    hipStream_t s = current_stream();
+    if (per_row) {
+        if (rows == 0)
+            return VTL_HIP_OK;
+        if (cols == 0)
+            return launch_fill_zero(absmax_out, rows, s);
+        const bool vec = (cols % 4 == 0) && aligned(x, 16);
+        if (vec && cols >= 4096)
+            hipLaunchKernelGGL((absmax_rows_kernel<256, 4>), dim3((unsigned)rows), dim3(256), 0, s, x,
+                               cols, absmax_out);
+        else if (vec)
+            hipLaunchKernelGGL((absmax_rows_kernel<64, 4>), dim3((unsigned)rows), dim3(64), 0, s, x,
+                               cols, absmax_out);
+        else
+            hipLaunchKernelGGL((absmax_rows_kernel<256, 1>), dim3((unsigned)rows), dim3(256), 0, s, x,
+                               cols, absmax_out);
+        return check_launch("absmax_rows_kernel");
+    }
+    st = launch_fill_zero(absmax_out, 1, s);
+    if (st != VTL_HIP_OK)
+        return st;
+    const int64_t n = rows * cols;
+    if (n == 0)
+        return VTL_HIP_OK;
+    const int vec_ok = aligned(x, 16) ? 1 : 0;
+    int64_t blocks = (n / 4 + 256 * 8 - 1) / (256 * 8);
+    if (blocks < 1)
+        blocks = 1;
+    if (blocks > 256 * 16)
+        blocks = 256 * 16;
+    hipLaunchKernelGGL((absmax_flat_kernel<256>), dim3((unsigned)blocks), dim3(256), 0, s, x, n, vec_ok,
+                       reinterpret_cast<unsigned *>(absmax_out));
+    return check_launch("absmax_flat_kernel");
+}
+
+int vtl_hip_quantize_with_scale_f32_i8(const float *x, const float *scale, int64_t rows,
+                                       int64_t cols, int per_row, int8_t *q)
+{
+    int st = check_2d(x, q, rows, cols);
+    if (st != VTL_HIP_OK)
+        return st;
+    if (!scale)
+        return VTL_HIP_ERR_INVALID_ARG;
+    if (rows == 0 || cols == 0)
+        return VTL_HIP_OK;
+    hipStream_t s = current_stream();
+    constexpr int T = 256, NV = 4;
+    if (per_row) {
+        const bool vec = (cols % 4 == 0) && aligned(x, 16) && aligned(q, 4);
+        const int64_t per_chunk = vec ? 4 * T * NV : T * NV;
+        const int64_t chunks = (cols + per_chunk - 1) / per_chunk;
+        if (chunks > kMaxGridY)
+            return VTL_HIP_ERR_UNSUPPORTED;
+        const dim3 grid((unsigned)rows, (unsigned)chunks);
+        if (vec)
+            hipLaunchKernelGGL((quantize_scaled_kernel<T, NV, 4>), grid, dim3(T), 0, s, x, scale, 1, cols,
+                               q);
+        else
+            hipLaunchKernelGGL((quantize_scaled_kernel<T, NV, 1>), grid, dim3(T), 0, s, x, scale, 1, cols,
+                               q);
+    } else {
+        const int64_t n = rows * cols;
+        const bool vec = aligned(x, 16) && aligned(q, 4);
+        const int64_t per_chunk = vec ? 4 * T * NV : T * NV;
+        const int64_t chunks = (n + per_chunk - 1) / per_chunk;
+        if (chunks > kMaxGridX)
+            return VTL_HIP_ERR_UNSUPPORTED;
+        const dim3 grid((unsigned)chunks);
+        if (vec)
+            hipLaunchKernelGGL((quantize_scaled_kernel<T, NV, 4>), grid, dim3(T), 0, s, x, scale, 0, n, q);
+        else
+            hipLaunchKernelGGL((quantize_scaled_kernel<T, NV, 1>), grid, dim3(T), 0, s, x, scale, 0, n, q);
+    }
+    return check_launch("quantize_scaled_kernel");
+}
+
+int vtl_hip_quantize_f32_i8(const float *x, int64_t rows, int64_t cols, int per_row, int8_t *q,
+                            float *scale_out)
+{
+    int st = check_2d(x, q, rows, cols);
+    if (st != VTL_HIP_OK)
+        return st;
+    if (!scale_out)
+        return VTL_HIP_ERR_INVALID_ARG;
+    hipStream_t s = current_stream();
+    if (per_row)
+        return launch_quantize_rows(x, rows, cols, q, scale_out, s);
+    // whole tensor: absmax pass, scale in place, then the scaled quantize pass
+    st = vtl_hip_absmax_f32(x, rows, cols, 0, scale_out);
+    if (st != VTL_HIP_OK)
+        return st;
+    hipLaunchKernelGGL(scale_from_absmax_kernel, dim3(1), dim3(64), 0, s, scale_out, (int64_t)1);
+    st = check_launch("scale_from_absmax_kernel");
+    if (st != VTL_HIP_OK)
+        return st;
+    return vtl_hip_quantize_with_scale_f32_i8(x, scale_out, rows, cols, 0, q);
+}
+
+int vtl_hip_dequantize_i8_f32(const int8_t *q, const float *scale, int64_t rows, int64_t cols,
+                              int per_row, float *x)
+{
+    int st = check_2d(q, x, rows, cols);
+    if (st != VTL_HIP_OK)
+        return st;
+    if (!scale)
+        return VTL_HIP_ERR_INVALID_ARG;
+    if (rows == 0 || cols == 0)
+        return VTL_HIP_OK;
+    hipStream_t s = current_stream();
+    constexpr int T = 256, NV = 4;
+    if (per_row) {
+        const bool vec = (cols % 4 == 0) && aligned(x, 16) && aligned(q, 4);
+        const int64_t per_chunk = vec ? 4 * T * NV : T * NV;
+        const int64_t chunks = (cols + per_chunk - 1) / per_chunk;
+        if (chunks > kMaxGridY)
+            return VTL_HIP_ERR_UNSUPPORTED;
+        const dim3 grid((unsigned)rows, (unsigned)chunks);
+        if (vec)
+            hipLaunchKernelGGL((dequantize_kernel<T, NV, 4>), grid, dim3(T), 0, s, q, scale, 1, cols, x);
+        else
+            hipLaunchKernelGGL((dequantize_kernel<T, NV, 1>), grid, dim3(T), 0, s, q, scale, 1, cols, x);
+    } else {
+        const int64_t n = rows * cols;
+        const bool vec = aligned(x, 16) && aligned(q, 4);
+        const int64_t per_chunk = vec ? 4 * T * NV : T * NV;
+        const int64_t chunks = (n + per_chunk - 1) / per_chunk;
+        if (chunks > kMaxGridX)
+            return VTL_HIP_ERR_UNSUPPORTED;
+        const dim3 grid((unsigned)chunks);
+        if (vec)
+            hipLaunchKernelGGL((dequantize_kernel<T, NV, 4>), grid, dim3(T), 0, s, q, scale, 0, n, x);
+        else
+            hipLaunchKernelGGL((dequantize_kernel<T, NV, 1>), grid, dim3(T), 0, s, q, scale, 0, n, x);
+    }
+    return check_launch("dequantize_kernel");
+}
+
+int vtl_hip_relu_f32(float *x, int64_t n)
+{
+    if (!x || n < 0)
+        return VTL_HIP_ERR_INVALID_ARG;
+    if (n == 0)
+        return VTL_HIP_OK;
+    const int64_t blocks = (n + 255) / 256;
+    if (blocks > kMaxGridX)
+        return VTL_HIP_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(relu_kernel, dim3((unsigned)blocks), dim3(256), 0, current_stream(), x, n);
+    return check_launch("relu_kernel");
+}
+
+}  // extern "C"

@@ -1,0 +1,213 @@
+// Device, memory, transfer, stream and timing entry points of libvtlhip.so.
+// These are the calls the V-side HipStorage makes where CudaStorage calls
+// cudaMalloc / cudaMemcpy / cudaFree (storage/cuda_d_cuda.v:32-102).
+#include <stdio.h>
+#include <string.h>
+
+#include "common.hpp"
+
+namespace vtlhip {
+
+static hipStream_t g_stream = nullptr;
+static thread_local char g_last_error[256] = "";
+
+hipStream_t current_stream() { return g_stream; }
+
+int record_hip_error(hipError_t e, const char *what)
+{
+    snprintf(g_last_error, sizeof(g_last_error), "%s: %s (%d)", what, hipGetErrorString(e), (int)e);
+    (void)hipGetLastError();  // clear the sticky per-thread error
+    if (e == hipErrorOutOfMemory)
+        return VTL_HIP_ERR_OUT_OF_MEMORY;
+    if (e == hipErrorNoDevice || e == hipErrorInvalidDevice)
+        return VTL_HIP_ERR_NO_DEVICE;
+    return VTL_HIP_ERR_RUNTIME;
+}
+
+int check_launch(const char *kernel_name)
+{
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess)
+        return record_hip_error(e, kernel_name);
+    return VTL_HIP_OK;
+}
+
+}  // namespace vtlhip
+
+using namespace vtlhip;
+
+extern "C" {
+
+int vtl_hip_device_count(int *n)
+{
+    if (!n)
+        return VTL_HIP_ERR_INVALID_ARG;
+    *n = 0;
+    int c = 0;
+    hipError_t e = hipGetDeviceCount(&c);
+    if (e != hipSuccess)
+        return record_hip_error(e, "hipGetDeviceCount");
+    *n = c;
+    return VTL_HIP_OK;
+}
+
+int vtl_hip_set_device(int device_id)
+{
+    int c = 0;
+    int st = vtl_hip_device_count(&c);
+    if (st != VTL_HIP_OK)
+        return st;
+    if (device_id < 0 || device_id >= c)
+        return VTL_HIP_ERR_NO_DEVICE;
+    VTL_HIP_TRY(hipSetDevice(device_id));
+    return VTL_HIP_OK;
+}
+
+int vtl_hip_device_info(char *name, size_t name_cap, int *compute_units, int *clock_mhz)
+{
+    int dev = 0;
+    VTL_HIP_TRY(hipGetDevice(&dev));
+    hipDeviceProp_t p;
+    VTL_HIP_TRY(hipGetDeviceProperties(&p, dev));
+    if (name && name_cap) {
+        snprintf(name, name_cap, "%s (%s)", p.name, p.gcnArchName);
+    }
+    if (compute_units)
+        *compute_units = p.multiProcessorCount;
+    if (clock_mhz)
+        *clock_mhz = p.clockRate / 1000;
+    return VTL_HIP_OK;
+}
+
+int vtl_hip_malloc(void **dptr, size_t bytes)
+{
+    if (!dptr || bytes == 0)
+        return VTL_HIP_ERR_INVALID_ARG;
+    *dptr = nullptr;
+    VTL_HIP_TRY(hipMalloc(dptr, bytes));
+    return VTL_HIP_OK;
+}
+
+int vtl_hip_free(void *dptr)
+{
+    if (!dptr)
+        return VTL_HIP_OK;  // CudaStorage.release() skips nil too
+    VTL_HIP_TRY(hipFree(dptr));
+    return VTL_HIP_OK;
+}
+
+int vtl_hip_memcpy_h2d(void *dst_device, const void *src_host, size_t bytes)
+{
+    if (bytes == 0)
+        return VTL_HIP_OK;
+    if (!dst_device || !src_host)
+        return VTL_HIP_ERR_INVALID_ARG;
+    VTL_HIP_TRY(hipMemcpyAsync(dst_device, src_host, bytes, hipMemcpyHostToDevice, current_stream()));
+    VTL_HIP_TRY(hipStreamSynchronize(current_stream()));
+    return VTL_HIP_OK;
+}
+
+int vtl_hip_memcpy_d2h(void *dst_host, const void *src_device, size_t bytes)
+{
+    if (bytes == 0)
+        return VTL_HIP_OK;
+    if (!dst_host || !src_device)
+        return VTL_HIP_ERR_INVALID_ARG;
+    VTL_HIP_TRY(hipMemcpyAsync(dst_host, src_device, bytes, hipMemcpyDeviceToHost, current_stream()));
+    VTL_HIP_TRY(hipStreamSynchronize(current_stream()));
+    return VTL_HIP_OK;
+}
+
+int vtl_hip_memcpy_d2d(void *dst_device, const void *src_device, size_t bytes)
+{
+    if (bytes == 0)
+        return VTL_HIP_OK;
+    if (!dst_device || !src_device)
+        return VTL_HIP_ERR_INVALID_ARG;
+    VTL_HIP_TRY(hipMemcpyAsync(dst_device, src_device, bytes, hipMemcpyDeviceToDevice, current_stream()));
+    return VTL_HIP_OK;
+}
+
+int vtl_hip_memset(void *dst_device, int byte_value, size_t bytes)
+{
+    if (bytes == 0)
+        return VTL_HIP_OK;
+    if (!dst_device)
+        return VTL_HIP_ERR_INVALID_ARG;
+    VTL_HIP_TRY(hipMemsetAsync(dst_device, byte_value, bytes, current_stream()));
+    return VTL_HIP_OK;
+}
+
+int vtl_hip_sync(void)
+{
+    VTL_HIP_TRY(hipStreamSynchronize(current_stream()));
+    return VTL_HIP_OK;
+}
+
+int vtl_hip_set_stream(void *hip_stream)
+{
+    g_stream = (hipStream_t)hip_stream;
+    return VTL_HIP_OK;
+}
+
+int vtl_hip_get_stream(void **hip_stream)
+{
+    if (!hip_stream)
+        return VTL_HIP_ERR_INVALID_ARG;
+    *hip_stream = (void *)g_stream;
+    return VTL_HIP_OK;
+}
+
+int vtl_hip_event_create(void **event)
+{
+    if (!event)
+        return VTL_HIP_ERR_INVALID_ARG;
+    hipEvent_t e;
+    VTL_HIP_TRY(hipEventCreate(&e));
+    *event = (void *)e;
+    return VTL_HIP_OK;
+}
+
+int vtl_hip_event_destroy(void *event)
+{
+    if (!event)
+        return VTL_HIP_OK;
+    VTL_HIP_TRY(hipEventDestroy((hipEvent_t)event));
+    return VTL_HIP_OK;
+}
+
+int vtl_hip_event_record(void *event)
+{
+    if (!event)
+        return VTL_HIP_ERR_INVALID_ARG;
+    VTL_HIP_TRY(hipEventRecord((hipEvent_t)event, current_stream()));
+    return VTL_HIP_OK;
+}
+
+int vtl_hip_event_elapsed_ms(void *start, void *stop, float *ms)
+{
+    if (!start || !stop || !ms)
+        return VTL_HIP_ERR_INVALID_ARG;
+    VTL_HIP_TRY(hipEventSynchronize((hipEvent_t)stop));
+    VTL_HIP_TRY(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+    return VTL_HIP_OK;
+}
+
+const char *vtl_hip_strerror(int status)
+{
+    switch (status) {
+    case VTL_HIP_OK: return "success";
+    case VTL_HIP_ERR_INVALID_ARG: return "invalid argument (null pointer, bad size or flag)";
+    case VTL_HIP_ERR_NO_DEVICE: return "no usable HIP device";
+    case VTL_HIP_ERR_RUNTIME: return "HIP runtime call failed";
+    case VTL_HIP_ERR_OUT_OF_MEMORY: return "out of device memory";
+    case VTL_HIP_ERR_UNSUPPORTED: return "shape not supported by the gfx950 kernels";
+    default: return "unknown status";
+    }
+}
+
+const char *vtl_hip_last_error(void) { return g_last_error; }
+
+const char *vtl_hip_version(void) { return "vtlhip 0.1 (gfx950)"; }
+
+}  // extern "C"

@@ -1,0 +1,214 @@
+"""Device tensor: the Python mirror of the V file `tensor_hip_d_hip.v`.
+
+Follows `CudaTensor[T]` (tensor_cuda_d_cuda.v:13-60): storage plus shape and
+row-major strides, `Tensor.hip()` / `.cpu()` / `.release()`, shape predicates,
+and the INT8 operations of the quantized-linear path.  numpy arrays stand in
+for `vtl.Tensor[T]` on the host side.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+from . import capi
+from .storage import HipParams, HipStorage
+
+
+def _strides_from_shape(shape):
+    """Row-major element strides (util.v:169-184)."""
+    strides = [1] * len(shape)
+    for i in range(len(shape) - 2, -1, -1):
+        strides[i] = strides[i + 1] * shape[i + 1]
+    return strides
+
+
+class HipTensor:
+    """`HipTensor[T]{data &storage.HipStorage[T]; memory; size; shape; strides}`."""
+
+    def __init__(self, data: HipStorage, shape):
+        self.data = data
+        self.memory = "row_major"
+        self.shape = [int(s) for s in shape]
+        self.size = int(np.prod(self.shape)) if self.shape else 1
+        self.strides = _strides_from_shape(self.shape)
+        if self.size != data.count:
+            raise ValueError(f"HipTensor: shape {self.shape} does not match {data.count} elements")
+
+    # -- construction / transfer (tensor_cuda_d_cuda.v:23-60) ----------------
+    @staticmethod
+    def from_host(t: np.ndarray, params: HipParams | None = None) -> "HipTensor":
+        """`(t &Tensor[T]) hip(params) !&HipTensor[T]`: row-major copy, then upload."""
+        row = np.ascontiguousarray(t)
+        return HipTensor(HipStorage.from_cpu(row, params), row.shape)
+
+    @staticmethod
+    def empty(shape, dtype, params: HipParams | None = None) -> "HipTensor":
+        count = int(np.prod(shape)) if len(shape) else 1
+        return HipTensor(HipStorage.empty(count, dtype, params), shape)
+
+    def hip(self, params: HipParams | None = None) -> "HipTensor":
+        return self
+
+    def cpu(self) -> np.ndarray:
+        return self.data.cpu().reshape(self.shape)
+
+    def release(self) -> None:
+        self.data.release()
+
+    # -- predicates (tensor_cuda_d_cuda.v:63-120) ------------------------------
+    @property
+    def dtype(self):
+        return self.data.dtype
+
+    @property
+    def ptr(self) -> int:
+        return self.data.ptr
+
+    def rank(self) -> int:
+        return len(self.shape)
+
+    def numel(self) -> int:
+        return self.size
+
+    def is_matrix(self) -> bool:
+        return self.rank() == 2
+
+    def is_square_matrix(self) -> bool:
+        return self.rank() == 2 and self.shape[0] == self.shape[1]
+
+    def is_vector(self) -> bool:
+        return self.rank() == 1
+
+    def is_row_major(self) -> bool:
+        return self.memory == "row_major"
+
+    def is_col_major(self) -> bool:
+        return self.memory == "col_major"
+
+    def _assert(self, dtype, matrix=True, what="tensor"):
+        if self.dtype != np.dtype(dtype):
+            raise TypeError(f"{what}: expected {np.dtype(dtype)}, got {self.dtype}")
+        if matrix and not self.is_matrix():
+            raise ValueError(f"{what}: Matrix expected, got shape {self.shape}")
+
+    # -- INT8 quantization vocabulary ------------------------------------------
+    def absmax(self, axis: int = -1) -> "HipTensor":
+        """max |x| over the tensor (axis -1) or per row (axis 0 keeps rows)."""
+        self._assert(np.float32, what="absmax")
+        rows, cols = self.shape
+        per_row = _per_row(axis)
+        out = HipTensor.empty([rows if per_row else 1], np.float32, HipParams(self.data.device_id))
+        capi.call("vtl_hip_absmax_f32", self.ptr, rows, cols, per_row, out.ptr)
+        return out
+
+    def quantize_i8(self, axis: int = -1):
+        """`quantize_i8(axis /*-1 tensor, 0 row*/) !(&HipTensor[i8], &HipTensor[f32])`."""
+        self._assert(np.float32, what="quantize_i8")
+        rows, cols = self.shape
+        per_row = _per_row(axis)
+        p = HipParams(self.data.device_id)
+        q = HipTensor.empty([rows, cols], np.int8, p)
+        s = HipTensor.empty([rows if per_row else 1], np.float32, p)
+        capi.call("vtl_hip_quantize_f32_i8", self.ptr, rows, cols, per_row, q.ptr, s.ptr)
+        return q, s
+
+    def quantize_i8_with_scale(self, scales: "HipTensor", axis: int = -1) -> "HipTensor":
+        self._assert(np.float32, what="quantize_i8_with_scale")
+        scales._assert(np.float32, matrix=False, what="scales")
+        rows, cols = self.shape
+        per_row = _per_row(axis)
+        if scales.size != (rows if per_row else 1):
+            raise ValueError(f"scales: expected {rows if per_row else 1} entries, got {scales.size}")
+        q = HipTensor.empty([rows, cols], np.int8, HipParams(self.data.device_id))
+        capi.call("vtl_hip_quantize_with_scale_f32_i8", self.ptr, scales.ptr, rows, cols, per_row, q.ptr)
+        return q
+
+    def dequantize(self, scales: "HipTensor", axis: int = -1) -> "HipTensor":
+        """`(q &HipTensor[i8]) dequantize(scales &HipTensor[f32], axis int) !&HipTensor[f32]`."""
+        self._assert(np.int8, what="dequantize")
+        scales._assert(np.float32, matrix=False, what="scales")
+        rows, cols = self.shape
+        per_row = _per_row(axis)
+        if scales.size != (rows if per_row else 1):
+            raise ValueError(f"scales: expected {rows if per_row else 1} entries, got {scales.size}")
+        x = HipTensor.empty([rows, cols], np.float32, HipParams(self.data.device_id))
+        capi.call("vtl_hip_dequantize_i8_f32", self.ptr, scales.ptr, rows, cols, per_row, x.ptr)
+        return x
+
+    def relu_(self) -> "HipTensor":
+        """In-place ReLU (x < 0 -> 0), cf. relu_cuda tensor_cuda_d_cuda.v:205-235."""
+        self._assert(np.float32, matrix=False, what="relu_")
+        capi.call("vtl_hip_relu_f32", self.ptr, self.size)
+        return self
+
+
+def _per_row(axis: int) -> int:
+    if axis == -1:
+        return 0
+    if axis == 0:
+        return 1
+    raise ValueError(f"axis {axis}: use -1 (whole tensor) or 0 (one scale per row)")
+
+
+def _matmul_shapes(a: HipTensor, bt: HipTensor):
+    """Shape rule of la.matmul (la/la.v:38-43) for a second operand stored [N,K]."""
+    if not a.is_matrix() or not bt.is_matrix():
+        raise ValueError("Matrix expected")
+    if a.shape[1] != bt.shape[1]:
+        raise ValueError(
+            f"Invalid shapes for matrix multiplication {a.shape} and {[bt.shape[1], bt.shape[0]]}")
+    return a.shape[0], bt.shape[0], a.shape[1]
+
+
+def gemm_i8_hip(dst: HipTensor, a: HipTensor, bt: HipTensor) -> None:
+    """`gemm_i8_hip(dst &HipTensor[int], a &HipTensor[i8], b &HipTensor[i8]) !`
+
+    dst[M,N] = a[M,K] . bt[N,K]^T in exact int32 (style of gemm_cuda,
+    tensor_cuda_d_cuda.v:155-177)."""
+    a._assert(np.int8, what="gemm_i8_hip a")
+    bt._assert(np.int8, what="gemm_i8_hip b")
+    dst._assert(np.int32, what="gemm_i8_hip dst")
+    M, N, K = _matmul_shapes(a, bt)
+    if dst.shape != [M, N]:
+        raise ValueError(f"gemm_i8_hip: dst shape {dst.shape}, expected {[M, N]}")
+    capi.call("vtl_hip_gemm_i8_i32", a.ptr, bt.ptr, dst.ptr, M, N, K)
+
+
+def linear_i8_hip(x_q: HipTensor, sx: HipTensor, w_q: HipTensor, sw: HipTensor,
+                  bias: HipTensor | None, relu: bool = False) -> HipTensor:
+    """`linear_i8_hip(x_q, sx, w_q, sw, bias) !&HipTensor[f32]`: y = x.W^T + b on int8 codes."""
+    x_q._assert(np.int8, what="linear_i8_hip x_q")
+    w_q._assert(np.int8, what="linear_i8_hip w_q")
+    M, N, K = _matmul_shapes(x_q, w_q)
+    if sx.size not in (1, M) or sw.size not in (1, N):
+        raise ValueError("linear_i8_hip: scale sizes do not match the operands")
+    if bias is not None and bias.size != N:
+        raise ValueError(f"linear_i8_hip: bias has {bias.size} entries, expected {N}")
+    y = HipTensor.empty([M, N], np.float32, HipParams(x_q.data.device_id))
+    capi.call("vtl_hip_linear_i8_f32", x_q.ptr, sx.ptr, int(sx.size == M), w_q.ptr, sw.ptr,
+              int(sw.size == N), bias.ptr if bias is not None else None, y.ptr, M, N, K, int(relu))
+    return y
+
+
+def linear_f32_dynquant_hip(x: HipTensor, w_q: HipTensor, sw: HipTensor, bias: HipTensor | None,
+                            relu: bool = False, workspace: HipStorage | None = None) -> HipTensor:
+    """Per-token quantization of x on the fly, then the int8 linear."""
+    x._assert(np.float32, what="linear_f32_dynquant_hip x")
+    w_q._assert(np.int8, what="linear_f32_dynquant_hip w_q")
+    M, N, K = _matmul_shapes(x, w_q)
+    if sw.size != N:
+        raise ValueError("linear_f32_dynquant_hip: one weight scale per output channel expected")
+    if bias is not None and bias.size != N:
+        raise ValueError(f"linear_f32_dynquant_hip: bias has {bias.size} entries, expected {N}")
+    need = int(capi.lib().vtl_hip_linear_f32_dynquant_workspace(M, K))
+    own = workspace is None or workspace.size < need
+    ws = HipStorage.empty(need, np.uint8, HipParams(x.data.device_id)) if own else workspace
+    y = HipTensor.empty([M, N], np.float32, HipParams(x.data.device_id))
+    try:
+        capi.call("vtl_hip_linear_f32_dynquant", x.ptr, w_q.ptr, sw.ptr,
+                  bias.ptr if bias is not None else None, y.ptr, M, N, K, int(relu), ws.ptr, ws.size)
+        if own:
+            capi.call("vtl_hip_sync")
+    finally:
+        if own:
+            ws.release()
+    return y
