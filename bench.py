@@ -1,0 +1,219 @@
+#!/usr/bin/env python3
+"""Benchmark of the INT8 quantized-linear path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one pass of the int8 Linear at M=N=K=4096 (int8 MFMA GEMM with the
+fused f32 scale/bias epilogue) over device-resident synthetic inputs.  The
+same run also times the per-row quantize and dequantize of a [16384,16384]
+f32 tensor (the bandwidth half of the metric) and the CPU oracle on a bounded
+sample of each workload.  Prints ONE JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+from vtl_amd import capi, workloads  # noqa: E402
+from vtl_amd.tensor import HipTensor  # noqa: E402
+
+METRIC = "int8 Linear TOPS @M=N=K=4096 + quant/dequant GB/s, % of MI355X roofline"
+PEAK_INT8_TOPS = 5000.0      # dense int8 MFMA, MI355X published
+PEAK_HBM_GBPS = 8000.0       # HBM3E, MI355X published
+
+
+class Timer:
+    """hipEvent pair recorded on the stream the kernels are launched on."""
+
+    def __init__(self):
+        self.e0, self.e1 = C.c_void_p(), C.c_void_p()
+        capi.call("vtl_hip_event_create", C.byref(self.e0))
+        capi.call("vtl_hip_event_create", C.byref(self.e1))
+
+    def run(self, fn, steps: int):
+        """Returns (wall seconds, device milliseconds) for `steps` calls of fn."""
+        capi.call("vtl_hip_sync")
+        t0 = time.perf_counter()
+        capi.call("vtl_hip_event_record", self.e0)
+        for _ in range(steps):
+            fn()
+        capi.call("vtl_hip_event_record", self.e1)
+        capi.call("vtl_hip_sync")
+        wall = time.perf_counter() - t0
+        ms = C.c_float()
+        capi.call("vtl_hip_event_elapsed_ms", self.e0, self.e1, C.byref(ms))
+        return wall, float(ms.value)
+
+
+def bench_linear(timer: Timer, steps: int, warmup: int, cpu: bool):
+    m = n = k = 4096
+    a, bt, sa, sb, bias = workloads.square_int8_gemm(m, n, k)
+    A, B = HipTensor.from_host(a), HipTensor.from_host(bt)
+    SA, SB, BIAS = HipTensor.from_host(sa), HipTensor.from_host(sb), HipTensor.from_host(bias)
+    Y = HipTensor.empty([m, n], np.float32)
+
+    def step():
+        capi.call("vtl_hip_linear_i8_f32", A.ptr, SA.ptr, 1, B.ptr, SB.ptr, 1, BIAS.ptr, Y.ptr, m, n, k, 0)
+
+    for _ in range(warmup):
+        step()
+    wall, dev_ms = timer.run(step, steps)
+    ops = 2.0 * m * n * k
+    kernel_ms = dev_ms / steps
+    res = {
+        "ms_per_step": wall * 1e3 / steps,
+        "tops": ops / (wall / steps) / 1e12,
+        "roofline": {"kernel": "gemm_i8_mfma_kernel (fused f32 epilogue)", "bound": "mfma",
+                     "achieved": ops / (kernel_ms * 1e-3) / 1e12, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+                     "frac": ops / (kernel_ms * 1e-3) / 1e12 / PEAK_INT8_TOPS,
+                     "kernel_us": kernel_ms * 1e3, "algorithmic_ops": ops, "traffic": None},
+    }
+    if cpu:
+        import oracle  # CPU baseline leg only
+        rows = 48      # bounded sample: 48 rows of A against the whole of Bt
+        t0 = time.perf_counter()
+        ref = oracle.linear_i8_f32(a[:rows], sa[:rows], bt, sb, bias, threads=1)
+        dt1 = time.perf_counter() - t0
+        threads = oracle.max_threads()
+        rows_mt = rows * min(threads, 16)
+        t0 = time.perf_counter()
+        oracle.linear_i8_f32(a[:rows_mt], sa[:rows_mt], bt, sb, bias, threads=threads)
+        dtn = time.perf_counter() - t0
+        got = Y.cpu()[:rows]
+        res["parity_sample_bit_exact"] = bool(np.array_equal(got, ref))
+        res["cpu_baseline"] = {"value": 2.0 * rows * n * k / dt1 / 1e12, "unit": "TOPS", "cores": 1,
+                               "kind": "port",
+                               "sample": f"{rows} of {m} rows of A against all of Bt, {dt1:.1f} s, 1 thread"}
+        res["cpu_baseline_all_cores"] = {"value": 2.0 * rows_mt * n * k / dtn / 1e12, "unit": "TOPS",
+                                         "cores": threads, "kind": "port",
+                                         "sample": f"{rows_mt} of {m} rows, {dtn:.1f} s, OpenMP"}
+    for h in (A, B, SA, SB, BIAS, Y):
+        h.release()
+    return res
+
+
+def bench_quant(timer: Timer, steps: int, warmup: int, cpu: bool):
+    rows = cols = 16384
+    x = workloads.outlier_matrix(rows, cols)
+    X = HipTensor.from_host(x)
+    Q = HipTensor.empty([rows, cols], np.int8)
+    S = HipTensor.empty([rows], np.float32)
+    D = HipTensor.empty([rows, cols], np.float32)
+    algo_bytes = rows * cols * 5.0 + rows * 4.0     # 4 B in + 1 B out (or 1 + 4) per element + scales
+    out = {}
+
+    def q_step():
+        capi.call("vtl_hip_quantize_f32_i8", X.ptr, rows, cols, 1, Q.ptr, S.ptr)
+
+    def d_step():
+        capi.call("vtl_hip_dequantize_i8_f32", Q.ptr, S.ptr, rows, cols, 1, D.ptr)
+
+    for name, fn, kern in (("quantize", q_step, "quantize_rows_reg_kernel<256,16>"),
+                           ("dequantize", d_step, "dequantize_kernel<256,4,4>")):
+        for _ in range(warmup):
+            fn()
+        wall, dev_ms = timer.run(fn, steps)
+        kernel_ms = dev_ms / steps
+        gbps = algo_bytes / (kernel_ms * 1e-3) / 1e9
+        out[name] = {
+            "value": algo_bytes / (wall / steps) / 1e9, "unit": "GB/s", "ms_per_step": wall * 1e3 / steps,
+            "config": {"workload": f"configs[1]: per-row {name} of f32 [16384,16384], seed 1"},
+            "roofline": {"kernel": kern, "bound": "hbm", "achieved": gbps, "peak": PEAK_HBM_GBPS,
+                         "unit": "GB/s", "frac": gbps / PEAK_HBM_GBPS, "kernel_us": kernel_ms * 1e3,
+                         "algorithmic_bytes": algo_bytes, "traffic": None},
+        }
+    if cpu:
+        import oracle  # CPU baseline leg only
+        sample = 1024   # rows
+        threads = oracle.max_threads()
+        t0 = time.perf_counter()
+        qr, sr = oracle.quantize(x[:sample], True, threads=1)
+        dq1 = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        dr = oracle.dequantize(qr, sr, True, threads=1)
+        dd1 = time.perf_counter() - t0
+        big = min(rows, sample * 8)
+        t0 = time.perf_counter()
+        oracle.quantize(x[:big], True, threads=threads)
+        dqn = time.perf_counter() - t0
+        sample_bytes = sample * cols * 5.0 + sample * 4.0
+        out["quantize"]["cpu_baseline"] = {"value": sample_bytes / dq1 / 1e9, "unit": "GB/s", "cores": 1,
+                                           "kind": "port", "sample": f"first {sample} rows, {dq1:.2f} s"}
+        out["quantize"]["cpu_baseline_all_cores"] = {
+            "value": (big * cols * 5.0 + big * 4.0) / dqn / 1e9, "unit": "GB/s", "cores": threads,
+            "kind": "port", "sample": f"first {big} rows, {dqn:.2f} s, OpenMP"}
+        out["dequantize"]["cpu_baseline"] = {"value": sample_bytes / dd1 / 1e9, "unit": "GB/s", "cores": 1,
+                                             "kind": "port", "sample": f"first {sample} rows, {dd1:.2f} s"}
+        out["quantize"]["parity_sample_bit_exact"] = bool(
+            np.array_equal(Q.cpu()[:sample], qr) and np.array_equal(S.cpu()[:sample], sr))
+        out["dequantize"]["parity_sample_bit_exact"] = bool(np.array_equal(D.cpu()[:sample], dr))
+    for h in (X, Q, S, D):
+        h.release()
+    return out
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only", choices=["all", "linear", "quant"], default="all")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus must be 1 "
+              "(the multi-GPU sharding is described in DESIGN.md, not built)", file=sys.stderr)
+        return 2
+    if capi.device_count() < 1:
+        print("bench.py: no HIP device visible", file=sys.stderr)
+        return 1
+    capi.call("vtl_hip_set_device", 0)
+    name, cus, mhz = capi.device_info()
+    timer = Timer()
+    cpu = not args.no_cpu_baseline
+
+    lin = bench_linear(timer, args.steps, args.warmup, cpu) if args.only in ("all", "linear") else None
+    qd = bench_quant(timer, args.steps, args.warmup, cpu) if args.only in ("all", "quant") else None
+
+    line = {
+        "metric": METRIC,
+        "value": lin["tops"] if lin else qd["quantize"]["value"],
+        "unit": "TOPS" if lin else "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": lin["ms_per_step"] if lin else qd["quantize"]["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "i8 (i32 accumulate, f32 epilogue)", "data": "synthetic",
+        "config": {"workload": ("configs[2]: int8 Linear M=N=K=4096, per-row x per-column f32 scales + bias, "
+                                "seed 2; secondary: configs[1] per-row quantize/dequantize of f32 "
+                                "[16384,16384], seed 1") if lin else qd["quantize"]["config"]["workload"],
+                   "device": name, "compute_units": cus, "clock_mhz": mhz},
+    }
+    if lin:
+        line["roofline"] = lin["roofline"]
+        if "cpu_baseline" in lin:
+            line["cpu_baseline"] = lin["cpu_baseline"]
+            line["cpu_baseline_all_cores"] = lin["cpu_baseline_all_cores"]
+            line["parity_sample_bit_exact"] = lin["parity_sample_bit_exact"]
+    elif qd:
+        line["roofline"] = qd["quantize"]["roofline"]
+        if "cpu_baseline" in qd["quantize"]:
+            line["cpu_baseline"] = qd["quantize"]["cpu_baseline"]
+    if qd:
+        line["quantize"] = qd["quantize"]
+        line["dequantize"] = qd["dequantize"]
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

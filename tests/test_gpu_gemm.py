@@ -1,0 +1,137 @@
+"""GPU parity of the int8 matmul and the fused f32 epilogue through the C ABI.
+
+Bar: int32 accumulators bit-exact; f32 outputs within 1e-5 relative of the
+oracle applying the same scales (the kernels keep the oracle's operation
+order, so equality is asserted as well).
+"""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import CPU_THREADS, KAT, dev, rel_err, raw_device_buffer, h2d, d2h
+from vtl_amd import capi, workloads
+from vtl_amd.tensor import HipTensor, gemm_i8_hip, linear_i8_hip
+
+pytestmark = pytest.mark.gpu
+
+F32_REL_TOL = 1e-5   # tolerance stated for dequantized f32 outputs
+
+
+def _gemm(a, bt):
+    A, B = dev(a), dev(bt)
+    Cm = HipTensor.empty([a.shape[0], bt.shape[0]], np.int32)
+    gemm_i8_hip(Cm, A, B)
+    out = Cm.cpu()
+    for h in (A, B, Cm):
+        h.release()
+    return out
+
+
+def test_identity_vector_from_reference_tests(hip):
+    v = KAT["reference_vocabulary"]["matmul_identity"]           # la/la_test.v:30-37
+    a = np.array(v["a"], np.int8)
+    b = np.array(v["b"], np.int8)
+    assert np.array_equal(_gemm(a, np.ascontiguousarray(b.T)), np.array(v["out"], np.int32))
+
+
+@pytest.mark.parametrize("k", KAT["gemm_closed_forms"]["k_values"])
+def test_closed_forms(hip, k):
+    ones = np.full((40, k), 127, np.int8)
+    assert np.all(_gemm(ones, ones) == k * 16129)
+    assert np.all(_gemm(ones, -ones) == -k * 16129)
+    alt = np.tile(np.array([1, -1], np.int8), k // 2)[None, :].repeat(5, 0)
+    assert np.all(_gemm(alt, np.ones((70, k), np.int8)) == 0)
+    n_eye = min(k, 96)
+    eye = np.eye(k, dtype=np.int8)[:n_eye] * 127
+    b = (np.arange(33 * k, dtype=np.int64).reshape(33, k) % 255 - 127)
+    assert np.array_equal(_gemm(eye, b.astype(np.int8)), 127 * b[:, :n_eye].T)
+
+
+def test_maximum_k_accumulates_without_overflow(hip):
+    k = 131072                                                   # K * 127^2 = 2 114 060 288 < 2^31
+    a = np.full((2, k), 127, np.int8)
+    assert np.all(_gemm(a, a) == k * 16129)
+    assert np.all(_gemm(a, -a) == -k * 16129)
+
+
+SHAPES = [(1, 1, 16), (1, 64, 4096), (8, 128, 256), (33, 65, 48), (17, 19, 23), (64, 256, 784),
+          (128, 128, 128), (256, 256, 128), (256, 512, 512), (300, 200, 144), (257, 255, 1040),
+          (512, 768, 384), (96, 11008 // 8, 640), (1024, 1024, 256), (5, 7, 1), (2, 3, 17)]
+
+
+@pytest.mark.parametrize("mnk", SHAPES)
+def test_gemm_and_linear_match_oracle(hip, mnk):
+    m, n, k = mnk
+    a, bt, sa, sb, bias = workloads.square_int8_gemm(m, n, k, seed=m * 31 + n * 17 + k)
+    ref = oracle.gemm_i8_i32(a, bt, threads=CPU_THREADS)
+    assert np.array_equal(_gemm(a, bt), ref)
+    A, B = dev(a), dev(bt)
+    for sa_v, sb_v, bias_v, relu in [(sa, sb, bias, False), (sa, sb, bias, True), (sa[:1], sb, None, False),
+                                     (sa, sb[:1], bias, True), (sa[:1], sb[:1], None, False)]:
+        dsa, dsb = dev(sa_v), dev(sb_v)
+        dbias = dev(bias_v) if bias_v is not None else None
+        y = linear_i8_hip(A, dsa, B, dsb, dbias, relu=relu)
+        got = y.cpu()
+        want = oracle.epilogue(ref, sa_v, sb_v, bias_v, relu=relu)
+        assert rel_err(got, want) <= F32_REL_TOL
+        assert np.array_equal(got, want)
+        for h in (dsa, dsb, y) + ((dbias,) if dbias is not None else ()):
+            h.release()
+    A.release()
+    B.release()
+
+
+def test_unaligned_operands_take_the_generic_kernel(hip):
+    a, bt, sa, sb, bias = workloads.square_int8_gemm(20, 24, 64, seed=5)
+    abuf, bbuf = raw_device_buffer(a.size + 64), raw_device_buffer(bt.size + 64)
+    cbuf = raw_device_buffer(20 * 24 * 4)
+    h2d(abuf.ptr + 3, a)
+    h2d(bbuf.ptr + 5, bt)
+    capi.call("vtl_hip_gemm_i8_i32", abuf.ptr + 3, bbuf.ptr + 5, cbuf.ptr, 20, 24, 64)
+    assert np.array_equal(d2h(cbuf.ptr, (20, 24), np.int32), oracle.gemm_i8_i32(a, bt))
+    for h in (abuf, bbuf, cbuf):
+        h.release()
+
+
+def test_shape_mismatch_is_reported_like_la_matmul(hip):
+    A, B = dev(np.zeros((4, 32), np.int8)), dev(np.zeros((6, 48), np.int8))
+    Cm = HipTensor.empty([4, 6], np.int32)
+    with pytest.raises(ValueError, match="Invalid shapes for matrix multiplication"):   # la/la.v:41-43
+        gemm_i8_hip(Cm, A, B)
+    with pytest.raises(ValueError, match="dst shape"):
+        gemm_i8_hip(HipTensor.empty([4, 5], np.int32), A, dev(np.zeros((6, 32), np.int8)))
+
+
+def test_square_gemm_config_full_size(hip):
+    """Config 3 at its real size 4096^3: full oracle parity on a band of rows,
+    exact row/column checksums and linearity over the whole product."""
+    m = n = k = 4096
+    a, bt, sa, sb, bias = workloads.square_int8_gemm(m, n, k)
+    A, B = dev(a), dev(bt)
+    Cm = HipTensor.empty([m, n], np.int32)
+    gemm_i8_hip(Cm, A, B)
+    c = Cm.cpu()
+    band = np.r_[0:96, 2000:2096, m - 64:m]
+    ref_band = oracle.gemm_i8_i32(a[band], bt, threads=CPU_THREADS)
+    assert np.array_equal(c[band], ref_band)
+    # checksums: 1^T C = (1^T A) B^T and C 1 = A (B^T 1), in int64
+    a64, b64 = a.astype(np.int64), bt.astype(np.int64)
+    assert np.array_equal(c.sum(axis=0, dtype=np.int64), a64.sum(axis=0) @ b64.T)
+    assert np.array_equal(c.sum(axis=1, dtype=np.int64), a64 @ b64.sum(axis=0))
+    # linearity in the second operand: C(A, B1 + B2) = C(A, B1) + C(A, B2)
+    b1 = (bt // 2).astype(np.int8)
+    b2 = (bt - b1).astype(np.int8)
+    B1, B2 = dev(b1), dev(b2)
+    C1, C2 = HipTensor.empty([m, n], np.int32), HipTensor.empty([m, n], np.int32)
+    gemm_i8_hip(C1, A, B1)
+    gemm_i8_hip(C2, A, B2)
+    assert np.array_equal(C1.cpu() + C2.cpu(), c)
+    # fused epilogue over the whole output against the oracle epilogue on the
+    # (already verified) accumulators
+    dsa, dsb, dbias = dev(sa), dev(sb), dev(bias)
+    y = linear_i8_hip(A, dsa, B, dsb, dbias).cpu()
+    want = oracle.epilogue(c, sa, sb, bias)
+    assert rel_err(y, want) <= F32_REL_TOL
+    assert np.array_equal(y, want)
+    for h in (A, B, Cm, B1, B2, C1, C2, dsa, dsb, dbias):
+        h.release()

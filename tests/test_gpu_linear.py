@@ -1,0 +1,135 @@
+"""GPU parity of the layer-level path (linear_forward_f32 hook, QuantLinearLayer,
+Sequential) on the benchmark configurations, through the host-side mirror."""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import CPU_THREADS, KAT, dev, rel_err
+from vtl_amd import (PER_CHANNEL, PER_TENSOR, HipSession, QuantLinearLayer, Sequential, capi,
+                     linear_forward_hip_f32, workloads)
+from vtl_amd.tensor import HipTensor, linear_f32_dynquant_hip
+
+pytestmark = pytest.mark.gpu
+
+F32_REL_TOL = 1e-5
+
+
+def _oracle_linear(x, w, bias, mode, relu=False):
+    per_row = mode == PER_CHANNEL
+    wq, sw = oracle.quantize(w, per_row, threads=CPU_THREADS)
+    xq, sx = oracle.quantize(x, per_row, threads=CPU_THREADS)
+    b = None if bias is None else np.asarray(bias, np.float32).reshape(-1)
+    return oracle.linear_i8_f32(xq, sx, wq, sw, b, relu=relu, threads=CPU_THREADS)
+
+
+def test_mnist_mlp_first_layer_config(hip, monkeypatch):
+    """Config 1: [64,784] x [256,784]^T, per-tensor scales, zero bias."""
+    monkeypatch.setenv("VTL_USE_HIP", "1")
+    x, w, b = workloads.mnist_mlp_first_layer()
+    got = linear_forward_hip_f32(x, w, b, mode=PER_TENSOR)
+    want = _oracle_linear(x, w, b, PER_TENSOR)
+    assert got.shape == (64, 256)
+    assert rel_err(got, want) <= F32_REL_TOL and np.array_equal(got, want)
+    # the int8 result tracks the reference's documented f32 Linear y = x.W^T + b
+    f32 = oracle.linear_f32_via_f64(x, w, b)
+    assert np.abs(got - f32).max() <= 0.02 * np.abs(f32).max()
+
+
+def test_tiny_linear_literals_from_reference_session_test(hip):
+    """x, W, b of autograd_cuda/device_session_test.v:34-36; y = [1.41, 3.22] in f32 math."""
+    v = KAT["reference_vocabulary"]["linear_f64_session"]
+    x, w, b = (np.array(v[k], np.float32) for k in ("x", "w", "b"))
+    layer = QuantLinearLayer(w, b, mode=PER_CHANNEL)
+    got = layer.forward(x)
+    assert got.shape == (1, 2)
+    assert np.array_equal(got, _oracle_linear(x, w, b, PER_CHANNEL))
+    assert np.allclose(got, np.array(v["out"], np.float32), rtol=0.02)   # int8 resolution
+    layer.release()
+
+
+@pytest.mark.parametrize("m", [1, 8, 32, 128])
+def test_decode_linear_config(hip, m):
+    """Config 4: K=4096, N=14336, per-output-channel weights, per-token activations."""
+    x, w = workloads.decode_linear(m)
+    wq, sw = oracle.quantize(w, True, threads=CPU_THREADS)
+    W = dev(w)
+    Wq, Sw = W.quantize_i8(0)
+    assert np.array_equal(Wq.cpu(), wq) and np.array_equal(Sw.cpu(), sw)
+    X = dev(x)
+    y = linear_f32_dynquant_hip(X, Wq, Sw, None)
+    got = y.cpu()
+    want = oracle.linear_f32_dynquant(x, wq, sw, None, threads=CPU_THREADS)
+    assert got.shape == (m, 14336)
+    assert rel_err(got, want) <= F32_REL_TOL and np.array_equal(got, want)
+    for h in (W, Wq, Sw, X, y):
+        h.release()
+
+
+def test_mlp_chain_config(hip):
+    """Config 5: 256x4096 -> 11008 -> ReLU -> 4096 -> ReLU -> 1024 through Sequential."""
+    x, ws = workloads.mlp_chain()
+    model = Sequential(mode=PER_CHANNEL).input([4096])
+    model.linear(11008, ws[0]).relu().linear(4096, ws[1]).relu().linear(1024, ws[2])
+    got = model.forward(x)
+    cur = x
+    for i, w in enumerate(ws):
+        cur = _oracle_linear(cur, w, np.zeros(w.shape[0], np.float32), PER_CHANNEL, relu=i < 2)
+    assert got.shape == (256, 1024)
+    assert rel_err(got, cur) <= F32_REL_TOL and np.array_equal(got, cur)
+    model.release()
+
+
+def test_sequential_builder_rules(hip):
+    with pytest.raises(ValueError):
+        Sequential().linear(4)                       # no input layer yet
+    model = Sequential(seed=3).input([48]).linear(32).relu().linear(16)
+    assert [l[0] for l in model.layers] == ["input", "linear", "relu", "linear"]
+    assert model.layers[1][1].weights.shape == (32, 48) and model.layers[3][1].weights.shape == (16, 32)
+    x = np.random.default_rng(0).standard_normal((5, 48)).astype(np.float32)
+    got = model.forward(x)
+    h = _oracle_linear(x, model.layers[1][1].weights, model.layers[1][1].bias, PER_CHANNEL, relu=True)
+    want = _oracle_linear(h, model.layers[3][1].weights, model.layers[3][1].bias, PER_CHANNEL)
+    assert np.array_equal(got, want)
+    with pytest.raises(ValueError, match="Invalid shapes"):
+        model.forward(np.zeros((2, 40), np.float32))
+    # a standalone ReLU layer (not preceded by a Linear) runs the ReLU kernel
+    m2 = Sequential().input([8]).relu()
+    assert np.array_equal(m2.forward(np.array([[-1, 2, -3, 4, 0, -0.5, 7, -8]], np.float32)),
+                          np.array([[0, 2, 0, 4, 0, 0, 7, 0]], np.float32))
+    model.release()
+
+
+def test_weight_cache_follows_parameter_replacement(hip):
+    rng = np.random.default_rng(1)
+    w1 = rng.standard_normal((8, 64)).astype(np.float32)
+    w2 = rng.standard_normal((8, 64)).astype(np.float32)
+    x = rng.standard_normal((3, 64)).astype(np.float32)
+    layer = QuantLinearLayer(w1)
+    y1 = layer.forward(x)
+    first = layer.quantized()
+    assert layer.quantized() is first                 # reused while the parameter is the same object
+    layer.weights = w2                                # optimizers assign a new tensor (adam.v:115,136)
+    y2 = layer.forward(x)
+    assert layer.quantized() is not first
+    assert np.array_equal(y1, _oracle_linear(x, w1, None, PER_CHANNEL))
+    assert np.array_equal(y2, _oracle_linear(x, w2, None, PER_CHANNEL))
+    layer.release()
+
+
+def test_session_reuses_buffers_on_second_forward(hip):
+    """cf. test_device_session_reuses_buffers_on_second_forward,
+    autograd_cuda/device_session_test.v:25-48."""
+    s = HipSession()
+    a = s.ensure("dynquant", 1000)
+    assert s.ensure("dynquant", 500) is a and s.ensure("dynquant", 1000) is a
+    b = s.ensure("dynquant", 5000)
+    assert b is not a and b.size >= 5000
+    rng = np.random.default_rng(2)
+    layer = QuantLinearLayer(rng.standard_normal((16, 128)).astype(np.float32))
+    X = dev(rng.standard_normal((4, 128)).astype(np.float32))
+    y1 = layer.forward_device(X, session=s).cpu()
+    buf = s.ensure("dynquant", 1)
+    y2 = layer.forward_device(X, session=s).cpu()
+    assert s.ensure("dynquant", 1) is buf and np.array_equal(y1, y2)
+    s.release()
+    layer.release()

@@ -1,0 +1,220 @@
+"""Linear layer on the INT8 HIP path: the Python mirror of the V files
+`nn/layers/hip_config.v`, `linear_hip_hooks_d_hip.v` and `linear_hip_d_hip.v`.
+
+The reference's f32 Linear is `y = x.W^T + b` with W stored
+`[out_features, in_features]` and bias `[1, out_features]`
+(nn/layers/linear.v:10-33); its backend hook is
+`linear_forward_f32` (nn/layers/linear_forward_f32.v:7-14), which asks
+`linear_forward_f32_use_<backend>()` and tries the device path.  This module
+adds the HIP branch of that hook.  The device path returns host tensors, like
+every GPU path of the reference (docs/DEVICE_MEMORY.md:9-16), unless the
+caller chains layers on the device explicitly (`forward_device`).
+
+There is no CPU arithmetic in here: a failing device call raises
+`capi.VtlHipError`.  (In V the hook site keeps the reference's own
+`or { return linear_forward_f32_cpu(...) }`, which is VTL's code, not this
+library's.)
+"""
+from __future__ import annotations
+
+import os
+
+import numpy as np
+
+from . import capi
+from .storage import HipParams, HipStorage
+from .tensor import HipTensor, linear_f32_dynquant_hip, linear_i8_hip
+
+
+# -- nn/layers/hip_config.v (cf. vulkan_config.v:12-24, cuda_config.v:11-23) ----
+
+def hip_linear_enabled() -> bool:
+    """True when the user opts in with VTL_USE_HIP=1 (and the build has `-d hip`)."""
+    return os.environ.get("VTL_USE_HIP") == "1"
+
+
+def hip_tests_enabled() -> bool:
+    """Gate for device tests, VTL_TEST_HIP=1 (cf. vulkan_tests_enabled)."""
+    return os.environ.get("VTL_TEST_HIP") == "1"
+
+
+def linear_forward_f32_use_hip() -> bool:
+    """Hook consulted by linear_forward_f32 (cf. linear_vulkan_hooks_d_vulkan.v:9)."""
+    return hip_linear_enabled()
+
+
+# -- quantization granularity ------------------------------------------------------
+
+PER_TENSOR = "per_tensor"      # one scale for x, one for W
+PER_CHANNEL = "per_channel"    # one scale per row of x (token) and per row of W (output channel)
+
+
+class HipSession:
+    """Reusable device buffers for one Context, cf. DeviceSession
+    (autograd_cuda/device_session.v:13-24) and GpuDevBuf.ensure
+    (autograd_cuda/device_session_gpu_d_cuda.v:24-39): a buffer grows when a
+    larger request arrives and is otherwise reused."""
+
+    def __init__(self, params: HipParams | None = None):
+        self.params = params or HipParams()
+        self._bufs: dict[str, HipStorage] = {}
+
+    def ensure(self, name: str, nbytes: int) -> HipStorage:
+        cur = self._bufs.get(name)
+        if cur is not None and cur.size >= nbytes:
+            return cur
+        if cur is not None:
+            cur.release()
+        buf = HipStorage.empty(max(int(nbytes), 256), np.uint8, self.params)
+        self._bufs[name] = buf
+        return buf
+
+    def release(self) -> None:
+        for b in self._bufs.values():
+            b.release()
+        self._bufs.clear()
+
+
+class QuantizedWeights:
+    """Device-resident int8 weights of one Linear layer, derived once from the
+    f32 parameter (the reference's optimizers assign a new tensor each step,
+    nn/optimizers/adam.v:115,136, so the cache is keyed on the array object)."""
+
+    def __init__(self, weights: np.ndarray, bias: np.ndarray | None, mode: str,
+                 params: HipParams | None = None):
+        if weights.ndim != 2:
+            raise ValueError("Matrix expected")
+        if mode not in (PER_TENSOR, PER_CHANNEL):
+            raise ValueError(f"unknown quantization mode {mode!r}")
+        self.mode = mode
+        self.source = weights
+        self.out_features, self.in_features = weights.shape
+        w_dev = HipTensor.from_host(np.asarray(weights, np.float32), params)
+        try:
+            self.w_q, self.sw = w_dev.quantize_i8(0 if mode == PER_CHANNEL else -1)
+        finally:
+            w_dev.release()
+        self.bias = None
+        if bias is not None:
+            b = np.asarray(bias, np.float32).reshape(-1)
+            if b.size != self.out_features:
+                raise ValueError(f"bias has {b.size} entries, expected {self.out_features}")
+            self.bias = HipTensor.from_host(b, params)
+
+    def release(self) -> None:
+        self.w_q.release()
+        self.sw.release()
+        if self.bias is not None:
+            self.bias.release()
+
+
+def linear_forward_hip_i8_device(x: HipTensor, qw: QuantizedWeights, relu: bool = False,
+                                 session: HipSession | None = None) -> HipTensor:
+    """x[M,K] f32 on the device -> y[M,N] f32 on the device."""
+    if not x.is_matrix():
+        raise ValueError("Matrix expected")
+    if x.shape[1] != qw.in_features:
+        raise ValueError(
+            f"Invalid shapes for matrix multiplication {x.shape} and {[qw.in_features, qw.out_features]}")
+    if qw.mode == PER_CHANNEL:
+        ws = None
+        if session is not None:
+            need = int(capi.lib().vtl_hip_linear_f32_dynquant_workspace(x.shape[0], x.shape[1]))
+            ws = session.ensure("dynquant", need)
+        return linear_f32_dynquant_hip(x, qw.w_q, qw.sw, qw.bias, relu=relu, workspace=ws)
+    x_q, sx = x.quantize_i8(-1)
+    try:
+        return linear_i8_hip(x_q, sx, qw.w_q, qw.sw, qw.bias, relu=relu)
+    finally:
+        capi.call("vtl_hip_sync")
+        x_q.release()
+        sx.release()
+
+
+def linear_forward_hip_f32(x: np.ndarray, weights: np.ndarray, bias: np.ndarray | None,
+                           mode: str = PER_CHANNEL) -> np.ndarray:
+    """`linear_forward_hip_f32(x, weights, bias) !&vtl.Tensor[f32]`: the HIP entry
+    of the f32 hook (cf. linear_forward_vulkan_f32, linear_vulkan_d_vulkan.v:7-12).
+    Uploads, quantizes both operands, runs the int8 linear, returns a host tensor."""
+    if not hip_linear_enabled():
+        raise RuntimeError("linear_forward_hip_f32: set VTL_USE_HIP=1 to enable")
+    return _linear_host_roundtrip(x, weights, bias, mode)
+
+
+def _linear_host_roundtrip(x, weights, bias, mode) -> np.ndarray:
+    x = np.asarray(x, np.float32)
+    if x.ndim != 2 or np.ndim(weights) != 2:
+        raise ValueError("Matrix expected")
+    qw = QuantizedWeights(weights, bias, mode)
+    x_dev = HipTensor.from_host(x)
+    try:
+        y = linear_forward_hip_i8_device(x_dev, qw)
+        try:
+            return y.cpu()
+        finally:
+            y.release()
+    finally:
+        x_dev.release()
+        qw.release()
+
+
+class QuantLinearLayer:
+    """`LinearLayer[f32]` (nn/layers/linear.v:17-74) whose forward runs on the
+    INT8 HIP path.  Parameters stay on the host as f32 (as in the reference);
+    the int8 copy is derived state, rebuilt when `weights` is replaced."""
+
+    def __init__(self, weights: np.ndarray, bias: np.ndarray | None = None, mode: str = PER_CHANNEL,
+                 params: HipParams | None = None):
+        weights = np.asarray(weights, np.float32)
+        if weights.ndim != 2:
+            raise ValueError("Matrix expected")
+        self.weights = weights                                   # [out, in]
+        self.bias = (np.zeros((1, weights.shape[0]), np.float32) if bias is None
+                     else np.asarray(bias, np.float32).reshape(1, -1))  # [1, out]
+        self.mode = mode
+        self.params = params or HipParams()
+        self._cache: QuantizedWeights | None = None
+
+    def output_shape(self):
+        return [self.weights.shape[0]]
+
+    def variables(self):
+        return [self.weights, self.bias]
+
+    def quantized(self) -> QuantizedWeights:
+        if self._cache is None or self._cache.source is not self.weights:
+            if self._cache is not None:
+                self._cache.release()
+            self._cache = QuantizedWeights(self.weights, self.bias, self.mode, self.params)
+        return self._cache
+
+    def forward_device(self, x: HipTensor, relu: bool = False,
+                       session: HipSession | None = None) -> HipTensor:
+        return linear_forward_hip_i8_device(x, self.quantized(), relu=relu, session=session)
+
+    def forward(self, x: np.ndarray) -> np.ndarray:
+        x = np.asarray(x, np.float32)
+        if x.ndim != 2:
+            raise ValueError("Matrix expected")
+        x_dev = HipTensor.from_host(x, self.params)
+        try:
+            y = self.forward_device(x_dev)
+            try:
+                return y.cpu()
+            finally:
+                y.release()
+        finally:
+            x_dev.release()
+
+    def release(self) -> None:
+        if self._cache is not None:
+            self._cache.release()
+            self._cache = None
+
+
+def kaiming_normal(shape, rng: np.random.Generator) -> np.ndarray:
+    """Weight initialiser of linear_layer (nn/layers/linear.v:25, nn/internal/init.v:21-70):
+    N(0, sqrt(2 / fan_in)) where compute_fans multiplies both fans by shape[1]."""
+    f0 = shape[0] * int(np.prod(shape[1:]))
+    std = np.sqrt(2.0 / f0)
+    return (rng.standard_normal(shape) * std).astype(np.float32)

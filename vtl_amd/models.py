@@ -1,0 +1,81 @@
+"""`Sequential` builder restricted to what the INT8 path needs: the Python
+mirror of nn/models/sequential.v:52-220 for input / linear / relu / forward.
+
+`linear(n)` takes its input width from the previous layer
+(nn/models/sequential_info.v:53-60); `forward` loops over the layers
+(sequential.v:204-215).  Between Linear layers the activations stay on the
+device and ReLU is folded into the producing Linear's epilogue, in the spirit
+of the reference's GPU activation chain
+(autograd_cuda/device_session_gpu_d_cuda.v:88-181).
+"""
+from __future__ import annotations
+
+import numpy as np
+
+from .layers import PER_CHANNEL, HipSession, QuantLinearLayer, kaiming_normal
+from .storage import HipParams
+from .tensor import HipTensor
+
+
+class Sequential:
+    def __init__(self, mode: str = PER_CHANNEL, seed: int = 0, params: HipParams | None = None):
+        self.mode = mode
+        self.params = params or HipParams()
+        self.rng = np.random.Generator(np.random.Philox(seed))
+        self.layers: list = []          # ("input", [k]) | ("linear", layer) | ("relu",)
+        self._width: int | None = None
+        self.session = HipSession(self.params)
+
+    def input(self, shape) -> "Sequential":
+        if len(shape) != 1:
+            raise ValueError("only flat inputs reach a Linear layer")
+        self._width = int(shape[0])
+        self.layers.append(("input", list(shape)))
+        return self
+
+    def linear(self, output_size: int, weights: np.ndarray | None = None,
+               bias: np.ndarray | None = None) -> "Sequential":
+        if self._width is None:
+            raise ValueError("Sequential.linear: add an input layer first")
+        if weights is None:
+            weights = kaiming_normal([output_size, self._width], self.rng)
+        weights = np.asarray(weights, np.float32)
+        if list(weights.shape) != [output_size, self._width]:
+            raise ValueError(f"weights {list(weights.shape)}, expected {[output_size, self._width]}")
+        self.layers.append(("linear", QuantLinearLayer(weights, bias, self.mode, self.params)))
+        self._width = output_size
+        return self
+
+    def relu(self) -> "Sequential":
+        self.layers.append(("relu",))
+        return self
+
+    def forward(self, x: np.ndarray) -> np.ndarray:
+        x = np.asarray(x, np.float32)
+        if x.ndim != 2:
+            raise ValueError("Matrix expected")
+        cur = HipTensor.from_host(x, self.params)
+        try:
+            i, n = 0, len(self.layers)
+            while i < n:
+                kind = self.layers[i][0]
+                if kind == "linear":
+                    fuse = i + 1 < n and self.layers[i + 1][0] == "relu"
+                    nxt = self.layers[i][1].forward_device(cur, relu=fuse, session=self.session)
+                    cur.release()
+                    cur = nxt
+                    i += 2 if fuse else 1
+                elif kind == "relu":
+                    cur.relu_()
+                    i += 1
+                else:
+                    i += 1
+            return cur.cpu()
+        finally:
+            cur.release()
+
+    def release(self) -> None:
+        for l in self.layers:
+            if l[0] == "linear":
+                l[1].release()
+        self.session.release()
