@@ -1,6 +1,7 @@
 // int8 x int8 -> int32 matmul with a fused f32 scale/bias/ReLU epilogue, for
-// gfx950 (CDNA4): LDS-tiled, v_mfma_i32_32x32x32_i8, accumulators kept in
-// registers until the epilogue, which converts and scales them in place.
+// gfx950 (CDNA4): LDS-tiled, v_mfma_i32_32x32x32_i8, operand tiles loaded from
+// global memory straight into LDS, accumulators kept in registers until the
+// epilogue, which converts and scales them in place.
 //
 // Operand layout: A[M,K] and Bt[N,K] are both K-contiguous, so both LDS tiles
 // are "rows of K bytes" and a lane's MFMA operand is 16 consecutive K bytes of
@@ -19,8 +20,10 @@ namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float f4 __attribute__((ext_vector_type(4)));
 
-constexpr int BK = 128;  // bytes of K per LDS tile row (8 chunks of 16 bytes)
+#define VTL_GPTR(p) ((const __attribute__((address_space(1))) void *)(p))
+#define VTL_LPTR(p) ((__attribute__((address_space(3))) void *)(p))
 
 struct GemmArgs {
     const int8_t *A;   // [M,K]
@@ -35,17 +38,284 @@ struct GemmArgs {
     int relu;
 };
 
-// LDS address of 16-byte chunk `chunk` of tile row `row`.  The chunk index is
-// XOR-swizzled with row bits so that the 16 lanes a ds_read_b128 serves per
-// cycle (16 consecutive rows, same logical chunk) fall into distinct banks.
-__device__ __forceinline__ int lds_off(int row, int chunk)
+// LDS tiles are rows of BK bytes (BK/16 chunks of 16 bytes).  The chunk index
+// is XOR-swizzled with row bits so that the 16 lanes a ds_read_b128 serves per
+// cycle (16 consecutive rows, same logical chunk) fall into 16 distinct
+// 16-byte bank groups of the 64-bank LDS.
+template <int BK>
+__device__ __forceinline__ int swizzle(int row)
 {
-    return row * BK + (((chunk ^ (row >> 1)) & 7) << 4);
+    return BK == 128 ? ((row >> 1) & 7) : ((row >> 2) & 3);
 }
 
-template <int BM, int BN, int WR, int WC, bool F32OUT, bool EDGE>
-__global__ __launch_bounds__(64 * WR * WC) void gemm_i8_mfma_kernel(const GemmArgs g)
+template <int BK>
+__device__ __forceinline__ int lds_off(int row, int chunk)
 {
+    return row * BK + (((chunk ^ swizzle<BK>(row)) & (BK / 16 - 1)) << 4);
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt()
+{
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// Workgroups are dealt round-robin to the 8 XCDs; renumber them so that each
+// XCD (own L2) works on a compact patch of the tile grid, then walk the grid
+// in groups of 8 tile rows.
+__device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int &tile_m, int &tile_n)
+{
+    const int total = tiles_m * tiles_n;
+    int pid = blockIdx.x;
+    if ((total & 7) == 0)
+        pid = (pid & 7) * (total >> 3) + (pid >> 3);
+    constexpr int GM = 8;
+    const int group_size = GM * tiles_n;
+    const int first_m = (pid / group_size) * GM;
+    const int gm = min(tiles_m - first_m, GM);
+    tile_m = first_m + (pid % group_size) % gm;
+    tile_n = (pid % group_size) / gm;
+}
+
+// Epilogue shared by the tiled kernels.  Accumulator register r of lane l of a
+// 32x32 MFMA tile holds row 8*(r/4) + 4*(l/32) + r%4, column l%32.  The scale
+// and bias slices of the block tile are staged in LDS (free once the K loop is
+// over); every output element is
+//     y = fl(fl(f32(acc) * fl(sa*sw)) + bias), then ReLU,
+// evaluated in that order with separately rounded operations.
+template <int BM, int BN, int WM, int WN, bool F32OUT, bool EDGE, int NT>
+__device__ __forceinline__ void epilogue(v16i (&acc)[WM / 32][WN / 32], const GemmArgs &g, int m0, int n0,
+                                         int wr, int wc, char *smem)
+{
+    constexpr int TM = WM / 32, TN = WN / 32;
+    const int lane = threadIdx.x & 63;
+    const int col_in = lane & 31, row_in = (lane >> 5) * 4;
+    const int M = g.M, N = g.N;
+    if constexpr (!F32OUT) {
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int n = n0 + wc * WN + j * 32 + col_in;
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int m = m0 + wr * WM + i * 32 + 8 * (r >> 2) + row_in + (r & 3);
+                    if (EDGE && (m >= M || n >= N))
+                        continue;
+                    reinterpret_cast<int32_t *>(g.out)[(int64_t)m * N + n] = acc[i][j][r];
+                }
+            }
+        }
+    } else {
+        float *s_sa = reinterpret_cast<float *>(smem);  // [BM]
+        float *s_sw = s_sa + BM;                        // [BN]
+        float *s_bias = s_sw + BN;                      // [BN]
+        __syncthreads();  // every wave is done with the operand tiles
+        for (int t = threadIdx.x; t < BM; t += NT) {
+            const int m = EDGE ? min(m0 + t, M - 1) : m0 + t;
+            s_sa[t] = g.sa[(int64_t)m * g.sa_stride];
+        }
+        for (int t = threadIdx.x; t < BN; t += NT) {
+            const int n = EDGE ? min(n0 + t, N - 1) : n0 + t;
+            s_sw[t] = g.sw[(int64_t)n * g.sw_stride];
+            s_bias[t] = g.bias ? g.bias[n] : 0.0f;
+        }
+        __syncthreads();
+        const bool has_bias = g.bias != nullptr;
+        const bool relu = g.relu != 0;
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int nl = wc * WN + j * 32 + col_in;
+            const int n = n0 + nl;
+            const float w = s_sw[nl];
+            const float bv = s_bias[nl];
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+#pragma unroll
+                for (int rq = 0; rq < 4; rq++) {
+                    const int ml = wr * WM + i * 32 + 8 * rq + row_in;
+                    const f4 a4 = *reinterpret_cast<const f4 *>(s_sa + ml);
+#pragma unroll
+                    for (int k = 0; k < 4; k++) {
+                        const int m = m0 + ml + k;
+                        if (EDGE && (m >= M || n >= N))
+                            continue;
+                        const float s = a4[k] * w;
+                        float y = (float)acc[i][j][rq * 4 + k] * s;
+                        if (has_bias)
+                            y = y + bv;
+                        if (relu && y < 0.0f)
+                            y = 0.0f;
+                        reinterpret_cast<float *>(g.out)[(int64_t)m * N + n] = y;
+                    }
+                }
+            }
+        }
+    }
+}
+
+// Main kernel.  Operand tiles go from global memory straight into LDS
+// (global_load_lds_dwordx4, no register staging): a wave instruction fills
+// 1 KiB of LDS in lane order, so the XOR swizzle is applied on the global side
+// (each lane fetches the chunk that belongs at its LDS slot).  NSTAGE tiles are
+// in flight.  MFMA operands are double-buffered in registers, and the
+// per-tile barrier sits before the last k-step of a tile so that its latency
+// and the first operand reads of the next tile hide behind that step's MFMAs.
+// Requires K % BK == 0; with EDGE, rows past M / N are clamped on load and
+// masked on store.
+template <int BM, int BN, int BK, int NSTAGE, int WR, int WC, bool F32OUT, bool EDGE>
+__global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArgs g)
+{
+    constexpr int NW = WR * WC, NT = 64 * NW;
+    constexpr int WM = BM / WR, WN = BN / WC, TM = WM / 32, TN = WN / 32;
+    constexpr int CPR = BK / 16;   // 16-byte chunks per tile row
+    constexpr int RPI = 64 / CPR;  // tile rows one wave instruction fills
+    constexpr int A_PW = BM / RPI / NW, B_PW = BN / RPI / NW;  // wave instructions per wave per tile
+    constexpr int LPT = A_PW + B_PW;
+    constexpr int KS = BK / 32;  // MFMA k-steps per tile
+    constexpr int STAGE = (BM + BN) * BK;
+    static_assert(KS % 2 == 0, "operand double buffering assumes an even number of k-steps");
+    static_assert(BM % (RPI * NW) == 0 && BN % (RPI * NW) == 0, "copy split");
+    static_assert(NSTAGE >= 2, "at least two stages");
+
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int M = g.M, N = g.N, K = g.K;
+    int tile_m, tile_n;
+    tile_of_block((M + BM - 1) / BM, (N + BN - 1) / BN, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int wr = w / WC, wc = w % WC;
+
+    // ---- global -> LDS ----
+    const int lrow = RPI * w + lane / CPR;                  // tile row of this lane for j = 0
+    const int lc = (lane % CPR) ^ swizzle<BK>(lrow);        // logical chunk it fetches (same for all j)
+    const int8_t *pa[EDGE ? A_PW : 1];
+    const int8_t *pb[EDGE ? B_PW : 1];
+    if constexpr (EDGE) {
+#pragma unroll
+        for (int j = 0; j < A_PW; j++)
+            pa[j] = g.A + (int64_t)min(m0 + lrow + j * RPI * NW, M - 1) * K + lc * 16;
+#pragma unroll
+        for (int j = 0; j < B_PW; j++)
+            pb[j] = g.Bt + (int64_t)min(n0 + lrow + j * RPI * NW, N - 1) * K + lc * 16;
+    } else {
+        pa[0] = g.A + (int64_t)(m0 + lrow) * K + lc * 16;
+        pb[0] = g.Bt + (int64_t)(n0 + lrow) * K + lc * 16;
+    }
+    const int64_t jstride = (int64_t)RPI * NW * K;
+    auto issue = [&](int kt, int st) {
+        char *sa_ = smem + st * STAGE;
+        char *sb_ = sa_ + BM * BK;
+        const int64_t ko = (int64_t)kt * BK;
+#pragma unroll
+        for (int j = 0; j < A_PW; j++)
+            __builtin_amdgcn_global_load_lds(VTL_GPTR(EDGE ? pa[EDGE ? j : 0] + ko : pa[0] + ko + j * jstride),
+                                             VTL_LPTR(sa_ + (w + NW * j) * 1024), 16, 0, 0);
+#pragma unroll
+        for (int j = 0; j < B_PW; j++)
+            __builtin_amdgcn_global_load_lds(VTL_GPTR(EDGE ? pb[EDGE ? j : 0] + ko : pb[0] + ko + j * jstride),
+                                             VTL_LPTR(sb_ + (w + NW * j) * 1024), 16, 0, 0);
+    };
+
+    v16i acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                acc[i][j][r] = 0;
+
+    // ---- LDS -> MFMA operands ----
+    const int frow = lane & 31;  // row inside a 32-row operand
+    const int fh = lane >> 5;    // which 16-byte half of the 32-byte k-step
+    int foff[KS];
+#pragma unroll
+    for (int s = 0; s < KS; s++)
+        foff[s] = lds_off<BK>(frow, 2 * s + fh);  // rows 32 apart share the swizzle
+    const int a_base = wr * WM * BK, b_base = BM * BK + wc * WN * BK;
+    v4i af[2][TM], bf[2][TN];
+    auto lfrag = [&](int st, int s, int buf) {
+        const char *sbase = smem + st * STAGE;
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+            af[buf][i] = *reinterpret_cast<const v4i *>(sbase + a_base + i * 32 * BK + foff[s]);
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+            bf[buf][j] = *reinterpret_cast<const v4i *>(sbase + b_base + j * 32 * BK + foff[s]);
+    };
+    auto mma = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[buf][i], bf[buf][j], acc[i][j], 0, 0, 0);
+    };
+    // scheduling hint: spread the TM+TN LDS reads of the next k-step between
+    // the TM*TN MFMAs of the current one
+    auto interleave = [&]() {
+        constexpr int NR = TM + TN, NM = TM * TN;
+        if constexpr (NM >= NR) {
+#pragma unroll
+            for (int r = 0; r < NR; r++) {
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);        // one LDS read
+                __builtin_amdgcn_sched_group_barrier(0x008, NM / NR, 0);  // MFMAs
+            }
+        }
+    };
+
+    const int KT = K / BK;
+#pragma unroll
+    for (int st = 0; st < NSTAGE; st++)
+        if (st < KT)
+            issue(st, st);
+    if (KT >= NSTAGE)
+        wait_vmcnt<(NSTAGE - 1) * LPT>();
+    else
+        wait_vmcnt<0>();
+    __builtin_amdgcn_s_barrier();
+    lfrag(0, 0, 0);
+    int st_c = 0;
+    for (int kt = 0; kt < KT - 1; kt++) {
+#pragma unroll
+        for (int s = 0; s < KS - 1; s++) {
+            lfrag(st_c, s + 1, (s + 1) & 1);
+            mma(s & 1);
+            interleave();
+        }
+        // every operand read of this tile has been issued: wait for them, make
+        // sure the next tile has landed, and hand this tile's buffer over
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        const int st_n = (st_c + 1 == NSTAGE) ? 0 : st_c + 1;
+        if (kt + NSTAGE - 1 < KT)
+            wait_vmcnt<(NSTAGE - 2) * LPT>();
+        else
+            wait_vmcnt<0>();
+        __builtin_amdgcn_s_barrier();
+        lfrag(st_n, 0, 0);
+        mma((KS - 1) & 1);
+        if (kt + NSTAGE < KT)
+            issue(kt + NSTAGE, st_c);
+        interleave();
+        st_c = st_n;
+    }
+#pragma unroll
+    for (int s = 0; s < KS - 1; s++) {
+        lfrag(st_c, s + 1, (s + 1) & 1);
+        mma(s & 1);
+        interleave();
+    }
+    mma((KS - 1) & 1);
+
+    epilogue<BM, BN, WM, WN, F32OUT, EDGE, NT>(acc, g, m0, n0, wr, wc, smem);
+}
+
+// Register-staged tile kernel for K that is a multiple of 16 but not of the
+// DMA kernel's tile depth: global -> VGPR -> LDS, zero-filled K tail.
+template <int BM, int BN, int WR, int WC, bool F32OUT>
+__global__ __launch_bounds__(64 * WR * WC) void gemm_i8_tile_kernel(const GemmArgs g)
+{
+    constexpr int BK = 128;
     constexpr int NT = 64 * WR * WC;
     constexpr int WM = BM / WR, WN = BN / WC;
     constexpr int TM = WM / 32, TN = WN / 32;
@@ -59,53 +329,28 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_mfma_kernel(const GemmAr
     char *sB = smem + 2 * BM * BK;  // [2][BN * BK]
 
     const int M = g.M, N = g.N, K = g.K;
-    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-    const int total = tiles_m * tiles_n;
-
-    // Workgroups are dealt round-robin to the 8 XCDs; renumber them so that
-    // each XCD (own L2) works on a compact patch of the tile grid.
-    int pid = blockIdx.x;
-    if ((total & 7) == 0)
-        pid = (pid & 7) * (total >> 3) + (pid >> 3);
-    constexpr int GM = 8;
-    const int group_size = GM * tiles_n;
-    const int first_m = (pid / group_size) * GM;
-    const int gm = min(tiles_m - first_m, GM);
-    const int tile_m = first_m + (pid % group_size) % gm;
-    const int tile_n = (pid % group_size) / gm;
+    int tile_m, tile_n;
+    tile_of_block((M + BM - 1) / BM, (N + BN - 1) / BN, tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wr = wave / WC, wc = wave % WC;
 
-    // ---- global -> register -> LDS copy assignment ----
     const int cc = tid & 7;   // 16-byte chunk inside the 128-byte row
     const int cr = tid >> 3;  // first row this thread copies
     v4i ra[A_CH], rb[B_CH];
-
     auto gload = [&](int kt) {
         const int kbyte = kt * BK + cc * 16;
 #pragma unroll
         for (int i = 0; i < A_CH; i++) {
-            int row = m0 + cr + i * ROWS_PER_PASS;
-            if (EDGE)
-                row = min(row, M - 1);
+            const int row = min(m0 + cr + i * ROWS_PER_PASS, M - 1);
             const v4i *p = reinterpret_cast<const v4i *>(g.A + (int64_t)row * K + kbyte);
-            if (EDGE)
-                ra[i] = (kbyte < K) ? *p : v4i{0, 0, 0, 0};
-            else
-                ra[i] = *p;
+            ra[i] = (kbyte < K) ? *p : v4i{0, 0, 0, 0};
         }
 #pragma unroll
         for (int i = 0; i < B_CH; i++) {
-            int row = n0 + cr + i * ROWS_PER_PASS;
-            if (EDGE)
-                row = min(row, N - 1);
+            const int row = min(n0 + cr + i * ROWS_PER_PASS, N - 1);
             const v4i *p = reinterpret_cast<const v4i *>(g.Bt + (int64_t)row * K + kbyte);
-            if (EDGE)
-                rb[i] = (kbyte < K) ? *p : v4i{0, 0, 0, 0};
-            else
-                rb[i] = *p;
+            rb[i] = (kbyte < K) ? *p : v4i{0, 0, 0, 0};
         }
     };
     auto lstore = [&](int buf) {
@@ -113,10 +358,10 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_mfma_kernel(const GemmAr
         char *b = sB + buf * (BN * BK);
 #pragma unroll
         for (int i = 0; i < A_CH; i++)
-            *reinterpret_cast<v4i *>(a + lds_off(cr + i * ROWS_PER_PASS, cc)) = ra[i];
+            *reinterpret_cast<v4i *>(a + lds_off<BK>(cr + i * ROWS_PER_PASS, cc)) = ra[i];
 #pragma unroll
         for (int i = 0; i < B_CH; i++)
-            *reinterpret_cast<v4i *>(b + lds_off(cr + i * ROWS_PER_PASS, cc)) = rb[i];
+            *reinterpret_cast<v4i *>(b + lds_off<BK>(cr + i * ROWS_PER_PASS, cc)) = rb[i];
     };
 
     v16i acc[TM][TN];
@@ -128,22 +373,21 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_mfma_kernel(const GemmAr
             for (int r = 0; r < 16; r++)
                 acc[i][j][r] = 0;
 
-    const int frow = lane & 31;  // row inside a 32-row MFMA operand
-    const int fch = lane >> 5;   // which 16-byte half of the 32-byte K step
-
+    const int frow = lane & 31;
+    const int fch = lane >> 5;
     auto compute = [&](int buf) {
-        const char *a = sA + buf * (BM * BK) + 0;
-        const char *b = sB + buf * (BN * BK) + 0;
+        const char *a = sA + buf * (BM * BK);
+        const char *b = sB + buf * (BN * BK);
 #pragma unroll
         for (int s = 0; s < BK / 32; s++) {
             v4i af[TM], bf[TN];
             const int ch = s * 2 + fch;
 #pragma unroll
             for (int i = 0; i < TM; i++)
-                af[i] = *reinterpret_cast<const v4i *>(a + lds_off(wr * WM + i * 32 + frow, ch));
+                af[i] = *reinterpret_cast<const v4i *>(a + lds_off<BK>(wr * WM + i * 32 + frow, ch));
 #pragma unroll
             for (int j = 0; j < TN; j++)
-                bf[j] = *reinterpret_cast<const v4i *>(b + lds_off(wc * WN + j * 32 + frow, ch));
+                bf[j] = *reinterpret_cast<const v4i *>(b + lds_off<BK>(wc * WN + j * 32 + frow, ch));
 #pragma unroll
             for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -165,43 +409,7 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_mfma_kernel(const GemmAr
             lstore((kt + 1) & 1);
         __syncthreads();
     }
-
-    // ---- epilogue: accumulator register r of lane l holds
-    //      row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its 32x32 tile ----
-    const int col_in = lane & 31;
-    const int row_in = (lane >> 5) * 4;
-#pragma unroll
-    for (int j = 0; j < TN; j++) {
-        const int n = n0 + wc * WN + j * 32 + col_in;
-        const bool n_ok = !EDGE || n < N;
-        float w = 0.f, bv = 0.f;
-        if (F32OUT && n_ok) {
-            w = g.sw[(int64_t)n * g.sw_stride];
-            if (g.bias)
-                bv = g.bias[n];
-        }
-#pragma unroll
-        for (int i = 0; i < TM; i++) {
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int m = m0 + wr * WM + i * 32 + 8 * (r >> 2) + row_in + (r & 3);
-                if (EDGE && !(n_ok && m < M))
-                    continue;
-                const int64_t o = (int64_t)m * N + n;
-                if (F32OUT) {
-                    const float s = g.sa[(int64_t)m * g.sa_stride] * w;
-                    float y = (float)acc[i][j][r] * s;
-                    if (g.bias)
-                        y = y + bv;
-                    if (g.relu && y < 0.0f)
-                        y = 0.0f;
-                    reinterpret_cast<float *>(g.out)[o] = y;
-                } else {
-                    reinterpret_cast<int32_t *>(g.out)[o] = acc[i][j][r];
-                }
-            }
-        }
-    }
+    epilogue<BM, BN, WM, WN, F32OUT, true, NT>(acc, g, m0, n0, wr, wc, smem);
 }
 
 // Any shape, any alignment: one output per thread.  Only used when K is not a
@@ -234,28 +442,41 @@ __global__ __launch_bounds__(256) void gemm_i8_naive_kernel(const GemmArgs g)
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-template <int BM, int BN, int WR, int WC, bool F32OUT, bool EDGE>
-int launch_tile(const GemmArgs &g, hipStream_t st)
+template <typename Kern>
+int launch_with_lds(Kern kern, bool &attr_done, int lds, int tiles, int threads, const GemmArgs &g,
+                    hipStream_t st, const char *name)
 {
-    auto kern = gemm_i8_mfma_kernel<BM, BN, WR, WC, F32OUT, EDGE>;
-    constexpr int lds = 2 * (BM + BN) * BK;
-    static bool attr_done = false;  // one host thread per device
-    if (!attr_done) {
+    if (!attr_done) {  // one host thread per device
         VTL_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds));
         attr_done = true;
     }
+    hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(threads), lds, st, g);
+    return check_launch(name);
+}
+
+template <int BM, int BN, int BK, int NSTAGE, int WR, int WC, bool F32OUT>
+int launch_dma(const GemmArgs &g, hipStream_t st)
+{
+    constexpr int lds = NSTAGE * (BM + BN) * BK;
+    static_assert(lds >= (BM + 2 * BN) * 4, "epilogue staging fits in the operand buffers");
     const int tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
-    hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(64 * WR * WC), lds, st, g);
-    return check_launch("gemm_i8_mfma_kernel");
+    static bool done_edge = false, done_full = false;
+    if ((g.M % BM) || (g.N % BN))
+        return launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, F32OUT, true>, done_edge, lds,
+                               tiles, 64 * WR * WC, g, st, "gemm_i8_dma_kernel");
+    return launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, F32OUT, false>, done_full, lds,
+                           tiles, 64 * WR * WC, g, st, "gemm_i8_dma_kernel");
 }
 
 template <int BM, int BN, int WR, int WC, bool F32OUT>
-int launch_tile_edge(const GemmArgs &g, hipStream_t st)
+int launch_tile(const GemmArgs &g, hipStream_t st)
 {
-    const bool edge = (g.M % BM) || (g.N % BN) || (g.K % BK);
-    return edge ? launch_tile<BM, BN, WR, WC, F32OUT, true>(g, st)
-                : launch_tile<BM, BN, WR, WC, F32OUT, false>(g, st);
+    constexpr int lds = 2 * (BM + BN) * 128;
+    const int tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
+    static bool done = false;
+    return launch_with_lds(gemm_i8_tile_kernel<BM, BN, WR, WC, F32OUT>, done, lds, tiles, 64 * WR * WC, g, st,
+                           "gemm_i8_tile_kernel");
 }
 
 template <bool F32OUT>
@@ -268,17 +489,23 @@ int launch_gemm(const GemmArgs &g, hipStream_t st)
         hipLaunchKernelGGL((gemm_i8_naive_kernel<F32OUT>), grid, dim3(256), 0, st, g);
         return check_launch("gemm_i8_naive_kernel");
     }
-    // Tile choice: the largest tile that still yields about one workgroup per
-    // compute unit; small problems trade tile efficiency for occupancy.
     const int64_t t256 = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256);
     const int64_t t128 = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
-    if (g.M > 128 && t256 >= 200)
-        return launch_tile_edge<256, 256, 2, 2, F32OUT>(g, st);
-    if (g.M > 64 && t128 >= 128)
-        return launch_tile_edge<128, 128, 2, 2, F32OUT>(g, st);
+    if (g.K % 128 == 0) {
+        // Largest tile that still gives most compute units a workgroup.
+        if (g.M > 128 && t256 >= 200)
+            return launch_dma<256, 256, 128, 2, 2, 4, F32OUT>(g, st);
+        if (g.M > 64)
+            return launch_dma<128, 128, 128, 2, 2, 2, F32OUT>(g, st);
+        if (g.M > 32)
+            return launch_dma<64, 128, 128, 2, 2, 2, F32OUT>(g, st);
+        return launch_dma<32, 128, 128, 2, 1, 4, F32OUT>(g, st);
+    }
+    if (g.M > 64 && t128 >= 64)
+        return launch_tile<128, 128, 2, 2, F32OUT>(g, st);
     if (g.M > 32)
-        return launch_tile_edge<64, 64, 2, 2, F32OUT>(g, st);
-    return launch_tile_edge<32, 64, 1, 2, F32OUT>(g, st);
+        return launch_tile<64, 64, 2, 2, F32OUT>(g, st);
+    return launch_tile<32, 64, 1, 2, F32OUT>(g, st);
 }
 
 int check_gemm_args(const void *A, const void *Bt, const void *out, int M, int N, int K)

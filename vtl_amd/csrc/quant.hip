@@ -262,16 +262,19 @@ __global__ __launch_bounds__(T) void quantize_rows_loop_kernel(const float *__re
 
 // ---- quantize with scales already on the device ----------------------------
 
-// per_row: block (x = row, y = chunk of the row); flat: block x = chunk of the
-// whole tensor.  A chunk is 4 * T * NV elements (VEC == 4) or T * NV (VEC == 1).
+// One workgroup per chunk of 4 * T * NV elements (VEC == 4) or T * NV
+// (VEC == 1).  The grid is one-dimensional and chunk-major (block = row *
+// chunks_per_row + chunk), so that workgroups dispatched back to back touch
+// adjacent memory; per_row == 0 treats the tensor as one row of `cols` elements.
 template <int T, int NV, int VEC>
 __global__ __launch_bounds__(T) void quantize_scaled_kernel(const float *__restrict__ x,
                                                             const float *__restrict__ scale,
                                                             int per_row, int64_t cols,
+                                                            unsigned chunks_per_row,
                                                             int8_t *__restrict__ q)
 {
-    const int64_t row = per_row ? (int64_t)blockIdx.x : 0;
-    const int64_t chunk = per_row ? (int64_t)blockIdx.y : (int64_t)blockIdx.x;
+    const int64_t row = per_row ? (int64_t)(blockIdx.x / chunks_per_row) : 0;
+    const int64_t chunk = per_row ? (int64_t)(blockIdx.x % chunks_per_row) : (int64_t)blockIdx.x;
     const float *xr = x + row * cols;
     int8_t *qr = q + row * cols;
     const QuantScale p = make_quant_scale(scale[row]);
@@ -311,15 +314,16 @@ __global__ __launch_bounds__(T) void quantize_scaled_kernel(const float *__restr
 
 // ---- dequantize -------------------------------------------------------------
 
-// Same block indexing as quantize_scaled_kernel.  Each lane reads four codes
+// Same chunk-major block indexing as quantize_scaled_kernel.  Each lane reads four codes
 // (4 bytes) and writes one 16-byte vector, so both sides stay coalesced.
 template <int T, int NV, int VEC>
 __global__ __launch_bounds__(T) void dequantize_kernel(const int8_t *__restrict__ q,
                                                        const float *__restrict__ scale, int per_row,
-                                                       int64_t cols, float *__restrict__ x)
+                                                       int64_t cols, unsigned chunks_per_row,
+                                                       float *__restrict__ x)
 {
-    const int64_t row = per_row ? (int64_t)blockIdx.x : 0;
-    const int64_t chunk = per_row ? (int64_t)blockIdx.y : (int64_t)blockIdx.x;
+    const int64_t row = per_row ? (int64_t)(blockIdx.x / chunks_per_row) : 0;
+    const int64_t chunk = per_row ? (int64_t)(blockIdx.x % chunks_per_row) : (int64_t)blockIdx.x;
     const int8_t *qr = q + row * cols;
     float *xr = x + row * cols;
     const float s = scale[row];
@@ -338,12 +342,12 @@ __global__ __launch_bounds__(T) void dequantize_kernel(const int8_t *__restrict_
         for (int i = 0; i < NV; i++) {
             const int64_t idx = base + i * T + threadIdx.x;
             if (idx < nv) {
-                const int w = (int)c[i];
+                const unsigned w = c[i];
                 float4_t o;
-                o.x = (float)((w << 24) >> 24) * s;
-                o.y = (float)((w << 16) >> 24) * s;
-                o.z = (float)((w << 8) >> 24) * s;
-                o.w = (float)(w >> 24) * s;
+                o.x = (float)((int)(w << 24) >> 24) * s;
+                o.y = (float)((int)(w << 16) >> 24) * s;
+                o.z = (float)((int)(w << 8) >> 24) * s;
+                o.w = (float)((int)w >> 24) * s;
                 __builtin_nontemporal_store(o, xv + idx);
             }
         }
@@ -377,7 +381,6 @@ __global__ __launch_bounds__(256) void relu_kernel(float *__restrict__ x, int64_
 inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
 constexpr int64_t kMaxGridX = 2147483647LL;
-constexpr int64_t kMaxGridY = 65535;
 
 int check_2d(const void *a, const void *b, int64_t rows, int64_t cols)
 {
@@ -418,12 +421,12 @@ int launch_quantize_rows(const float *x, int64_t rows, int64_t cols, int8_t *q, 
                        scale_out)
     if (vec && cols <= 4 * 64 * 1)
         VTL_Q_REG(64, 1);
-    else if (vec && cols <= 4 * 64 * 4)
-        VTL_Q_REG(64, 4);
-    else if (vec && cols <= 4 * 256 * 4)
-        VTL_Q_REG(256, 4);
-    else if (vec && cols <= 4 * 256 * 16)
-        VTL_Q_REG(256, 16);
+    else if (vec && cols <= 4 * 256 * 1)
+        VTL_Q_REG(256, 1);
+    else if (vec && cols <= 4 * 1024 * 1)
+        VTL_Q_REG(1024, 1);
+    else if (vec && cols <= 4 * 1024 * 4)
+        VTL_Q_REG(1024, 4);
     else if (vec && cols <= 4 * 1024 * 16)
         VTL_Q_REG(1024, 16);
     else if (vec)
@@ -491,33 +494,21 @@ int vtl_hip_quantize_with_scale_f32_i8(const float *x, const float *scale, int64
     if (rows == 0 || cols == 0)
         return VTL_HIP_OK;
     hipStream_t s = current_stream();
-    constexpr int T = 256, NV = 4;
-    if (per_row) {
-        const bool vec = (cols % 4 == 0) && aligned(x, 16) && aligned(q, 4);
-        const int64_t per_chunk = vec ? 4 * T * NV : T * NV;
-        const int64_t chunks = (cols + per_chunk - 1) / per_chunk;
-        if (chunks > kMaxGridY)
-            return VTL_HIP_ERR_UNSUPPORTED;
-        const dim3 grid((unsigned)rows, (unsigned)chunks);
-        if (vec)
-            hipLaunchKernelGGL((quantize_scaled_kernel<T, NV, 4>), grid, dim3(T), 0, s, x, scale, 1, cols,
-                               q);
-        else
-            hipLaunchKernelGGL((quantize_scaled_kernel<T, NV, 1>), grid, dim3(T), 0, s, x, scale, 1, cols,
-                               q);
-    } else {
-        const int64_t n = rows * cols;
-        const bool vec = aligned(x, 16) && aligned(q, 4);
-        const int64_t per_chunk = vec ? 4 * T * NV : T * NV;
-        const int64_t chunks = (n + per_chunk - 1) / per_chunk;
-        if (chunks > kMaxGridX)
-            return VTL_HIP_ERR_UNSUPPORTED;
-        const dim3 grid((unsigned)chunks);
-        if (vec)
-            hipLaunchKernelGGL((quantize_scaled_kernel<T, NV, 4>), grid, dim3(T), 0, s, x, scale, 0, n, q);
-        else
-            hipLaunchKernelGGL((quantize_scaled_kernel<T, NV, 1>), grid, dim3(T), 0, s, x, scale, 0, n, q);
-    }
+    constexpr int T = 512, NV = 2;
+    const int64_t row_len = per_row ? cols : rows * cols;
+    const bool vec = aligned(x, 16) && aligned(q, 4) && (!per_row || cols % 4 == 0);
+    const int64_t per_chunk = vec ? 4 * T * NV : T * NV;
+    const int64_t chunks = (row_len + per_chunk - 1) / per_chunk;
+    const int64_t blocks = per_row ? rows * chunks : chunks;
+    if (chunks > kMaxGridX || blocks > kMaxGridX)
+        return VTL_HIP_ERR_UNSUPPORTED;
+    const dim3 grid((unsigned)blocks);
+    if (vec)
+        hipLaunchKernelGGL((quantize_scaled_kernel<T, NV, 4>), grid, dim3(T), 0, s, x, scale,
+                           per_row ? 1 : 0, row_len, (unsigned)chunks, q);
+    else
+        hipLaunchKernelGGL((quantize_scaled_kernel<T, NV, 1>), grid, dim3(T), 0, s, x, scale,
+                           per_row ? 1 : 0, row_len, (unsigned)chunks, q);
     return check_launch("quantize_scaled_kernel");
 }
 
@@ -554,31 +545,23 @@ int vtl_hip_dequantize_i8_f32(const int8_t *q, const float *scale, int64_t rows,
     if (rows == 0 || cols == 0)
         return VTL_HIP_OK;
     hipStream_t s = current_stream();
-    constexpr int T = 256, NV = 4;
-    if (per_row) {
-        const bool vec = (cols % 4 == 0) && aligned(x, 16) && aligned(q, 4);
-        const int64_t per_chunk = vec ? 4 * T * NV : T * NV;
-        const int64_t chunks = (cols + per_chunk - 1) / per_chunk;
-        if (chunks > kMaxGridY)
-            return VTL_HIP_ERR_UNSUPPORTED;
-        const dim3 grid((unsigned)rows, (unsigned)chunks);
-        if (vec)
-            hipLaunchKernelGGL((dequantize_kernel<T, NV, 4>), grid, dim3(T), 0, s, q, scale, 1, cols, x);
-        else
-            hipLaunchKernelGGL((dequantize_kernel<T, NV, 1>), grid, dim3(T), 0, s, q, scale, 1, cols, x);
-    } else {
-        const int64_t n = rows * cols;
-        const bool vec = aligned(x, 16) && aligned(q, 4);
-        const int64_t per_chunk = vec ? 4 * T * NV : T * NV;
-        const int64_t chunks = (n + per_chunk - 1) / per_chunk;
-        if (chunks > kMaxGridX)
-            return VTL_HIP_ERR_UNSUPPORTED;
-        const dim3 grid((unsigned)chunks);
-        if (vec)
-            hipLaunchKernelGGL((dequantize_kernel<T, NV, 4>), grid, dim3(T), 0, s, q, scale, 0, n, x);
-        else
-            hipLaunchKernelGGL((dequantize_kernel<T, NV, 1>), grid, dim3(T), 0, s, q, scale, 0, n, x);
-    }
+    // Write-dominated: small chunk-major workgroups (16 KiB of output each) keep
+    // the stores of workgroups in flight adjacent in memory; measured best.
+    constexpr int T = 512, NV = 2;
+    const int64_t row_len = per_row ? cols : rows * cols;
+    const bool vec = aligned(x, 16) && aligned(q, 4) && (!per_row || cols % 4 == 0);
+    const int64_t per_chunk = vec ? 4 * T * NV : T * NV;
+    const int64_t chunks = (row_len + per_chunk - 1) / per_chunk;
+    const int64_t blocks = per_row ? rows * chunks : chunks;
+    if (chunks > kMaxGridX || blocks > kMaxGridX)
+        return VTL_HIP_ERR_UNSUPPORTED;
+    const dim3 grid((unsigned)blocks);
+    if (vec)
+        hipLaunchKernelGGL((dequantize_kernel<T, NV, 4>), grid, dim3(T), 0, s, q, scale, per_row ? 1 : 0,
+                           row_len, (unsigned)chunks, x);
+    else
+        hipLaunchKernelGGL((dequantize_kernel<T, NV, 1>), grid, dim3(T), 0, s, q, scale, per_row ? 1 : 0,
+                           row_len, (unsigned)chunks, x);
     return check_launch("dequantize_kernel");
 }
 
