@@ -31,6 +31,11 @@ METRIC = "int8 Linear TOPS @M=N=K=4096 + quant/dequant GB/s, % of MI355X rooflin
 PEAK_INT8_TOPS = 5000.0      # dense int8 MFMA, MI355X published
 PEAK_HBM_GBPS = 8000.0       # HBM3E, MI355X published
 
+# HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# script, each counter scaled by its reading for the 1 GiB copy_kernel (x2.000 and
+# x0.999); figures and commands in profiles/bench_pmc_traffic.md.
+PMC_TRAFFIC_BYTES = {"linear": 178.6e6, "quantize": 1342.6e6, "dequantize": 1342.7e6}
+
 
 class Timer:
     """hipEvent pair recorded on the stream the kernels are launched on."""
@@ -73,19 +78,20 @@ def bench_linear(timer: Timer, steps: int, warmup: int, cpu: bool):
     res = {
         "ms_per_step": wall * 1e3 / steps,
         "tops": ops / (wall / steps) / 1e12,
-        "roofline": {"kernel": "gemm_i8_mfma_kernel (fused f32 epilogue)", "bound": "mfma",
+        "roofline": {"kernel": "gemm_i8_dma_kernel<256,256,128,2,2,4,f32 epilogue>", "bound": "mfma",
                      "achieved": ops / (kernel_ms * 1e-3) / 1e12, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                      "frac": ops / (kernel_ms * 1e-3) / 1e12 / PEAK_INT8_TOPS,
-                     "kernel_us": kernel_ms * 1e3, "algorithmic_ops": ops, "traffic": None},
+                     "kernel_us": kernel_ms * 1e3, "algorithmic_ops": ops,
+                     "traffic": PMC_TRAFFIC_BYTES["linear"]},
     }
     if cpu:
         import oracle  # CPU baseline leg only
-        rows = 48      # bounded sample: 48 rows of A against the whole of Bt
+        rows = m       # the whole workload once: a few seconds on one host core
         t0 = time.perf_counter()
         ref = oracle.linear_i8_f32(a[:rows], sa[:rows], bt, sb, bias, threads=1)
         dt1 = time.perf_counter() - t0
         threads = oracle.max_threads()
-        rows_mt = rows * min(threads, 16)
+        rows_mt = m
         t0 = time.perf_counter()
         oracle.linear_i8_f32(a[:rows_mt], sa[:rows_mt], bt, sb, bias, threads=threads)
         dtn = time.perf_counter() - t0
@@ -118,8 +124,8 @@ def bench_quant(timer: Timer, steps: int, warmup: int, cpu: bool):
     def d_step():
         capi.call("vtl_hip_dequantize_i8_f32", Q.ptr, S.ptr, rows, cols, 1, D.ptr)
 
-    for name, fn, kern in (("quantize", q_step, "quantize_rows_reg_kernel<256,16>"),
-                           ("dequantize", d_step, "dequantize_kernel<256,4,4>")):
+    for name, fn, kern in (("quantize", q_step, "quantize_rows_reg_kernel<1024,4>"),
+                           ("dequantize", d_step, "dequantize_kernel<512,2,4>")):
         for _ in range(warmup):
             fn()
         wall, dev_ms = timer.run(fn, steps)
@@ -130,11 +136,11 @@ def bench_quant(timer: Timer, steps: int, warmup: int, cpu: bool):
             "config": {"workload": f"configs[1]: per-row {name} of f32 [16384,16384], seed 1"},
             "roofline": {"kernel": kern, "bound": "hbm", "achieved": gbps, "peak": PEAK_HBM_GBPS,
                          "unit": "GB/s", "frac": gbps / PEAK_HBM_GBPS, "kernel_us": kernel_ms * 1e3,
-                         "algorithmic_bytes": algo_bytes, "traffic": None},
+                         "algorithmic_bytes": algo_bytes, "traffic": PMC_TRAFFIC_BYTES[name]},
         }
     if cpu:
         import oracle  # CPU baseline leg only
-        sample = 1024   # rows
+        sample = rows   # the whole tensor once: under a second per pass on one host core
         threads = oracle.max_threads()
         t0 = time.perf_counter()
         qr, sr = oracle.quantize(x[:sample], True, threads=1)
@@ -142,7 +148,7 @@ def bench_quant(timer: Timer, steps: int, warmup: int, cpu: bool):
         t0 = time.perf_counter()
         dr = oracle.dequantize(qr, sr, True, threads=1)
         dd1 = time.perf_counter() - t0
-        big = min(rows, sample * 8)
+        big = rows
         t0 = time.perf_counter()
         oracle.quantize(x[:big], True, threads=threads)
         dqn = time.perf_counter() - t0
@@ -162,13 +168,35 @@ def bench_quant(timer: Timer, steps: int, warmup: int, cpu: bool):
     return out
 
 
+def bench_copy_calibration(timer: Timer, steps: int, warmup: int):
+    """Plain device-to-device copy of 1 GiB with the library's copy kernel: the
+    kernel of known traffic (1 GiB read + 1 GiB written per launch) that the
+    FETCH_SIZE / WRITE_SIZE hardware counters are scaled against."""
+    nbytes = 1 << 30
+    src = HipTensor.empty([nbytes // 4], np.float32)
+    dst = HipTensor.empty([nbytes // 4], np.float32)
+    capi.call("vtl_hip_memset", src.ptr, 1, nbytes)
+
+    def step():
+        capi.call("vtl_hip_memcpy_d2d", dst.ptr, src.ptr, nbytes)
+
+    for _ in range(warmup):
+        step()
+    wall, dev_ms = timer.run(step, steps)
+    gbps = 2.0 * nbytes / (dev_ms / steps * 1e-3) / 1e9
+    for h in (src, dst):
+        h.release()
+    return {"kernel": "copy_kernel", "bytes_read": nbytes, "bytes_written": nbytes,
+            "kernel_us": dev_ms / steps * 1e3, "GB/s": gbps}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["all", "linear", "quant"], default="all")
+    ap.add_argument("--only", choices=["all", "linear", "quant", "copy"], default="all")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 "
@@ -181,6 +209,9 @@ def main() -> int:
     name, cus, mhz = capi.device_info()
     timer = Timer()
     cpu = not args.no_cpu_baseline
+    if args.only == "copy":
+        print(json.dumps({"calibration": bench_copy_calibration(timer, args.steps, args.warmup)}))
+        return 0
 
     lin = bench_linear(timer, args.steps, args.warmup, cpu) if args.only in ("all", "linear") else None
     qd = bench_quant(timer, args.steps, args.warmup, cpu) if args.only in ("all", "quant") else None

@@ -1,0 +1,124 @@
+// Exercises the C++ host mirror (vtl_amd/host/vtl_hip.hpp) against the CPU
+// oracle on a real device: alloc -> H2D -> op -> D2H -> release, plus the error
+// paths.  Links libvtlhip.so (product) and libvtloracle.so (checker).
+// Exit code 0 = all checks passed.
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <random>
+
+#include "vtl_hip.hpp"
+#include "vtl_oracle.h"
+
+static int failures = 0;
+#define CHECK(cond)                                                        \
+    do {                                                                   \
+        if (!(cond)) {                                                     \
+            std::printf("FAIL %s:%d: %s\n", __FILE__, __LINE__, #cond);    \
+            failures++;                                                    \
+        }                                                                  \
+    } while (0)
+
+int main(int argc, char **argv)
+{
+    const bool no_device = argc > 1 && !std::strcmp(argv[1], "--no-device");
+    // error paths that need no device
+    CHECK(vtl_hip_quantize_f32_i8(nullptr, 1, 1, 1, nullptr, nullptr) == VTL_HIP_ERR_INVALID_ARG);
+    CHECK(vtl_hip_free(nullptr) == VTL_HIP_OK);
+    try {
+        vtl::per_row_of(3);
+        CHECK(false);
+    } catch (const std::invalid_argument &) {
+    }
+    try {
+        int m, n, k;
+        vtl::matmul_shapes({4, 32}, {6, 48}, m, n, k);
+        CHECK(false);
+    } catch (const std::invalid_argument &e) {
+        CHECK(std::strstr(e.what(), "Invalid shapes for matrix multiplication"));
+    }
+    if (no_device) {
+        std::printf(failures ? "host mirror: %d failure(s)\n" : "host mirror (no device): ok\n", failures);
+        return failures ? 1 : 0;
+    }
+
+    int ndev = 0;
+    CHECK(vtl_hip_device_count(&ndev) == VTL_HIP_OK && ndev > 0);
+    if (ndev <= 0)
+        return 1;
+    try {
+        vtl::HipStorage<float> bad(4, vtl::HipParams{ndev + 7});
+        CHECK(false);
+    } catch (const vtl::HipError &e) {
+        CHECK(e.status == VTL_HIP_ERR_NO_DEVICE);
+    }
+
+    std::mt19937 rng(1234);
+    std::normal_distribution<float> nd(0.f, 1.f);
+    const int M = 37, K = 256, N = 96;
+    std::vector<float> x((size_t)M * K), w((size_t)N * K), b(N);
+    for (auto &v : x) v = nd(rng);
+    for (auto &v : w) v = nd(rng) * 0.02f;
+    for (auto &v : b) v = nd(rng) * 0.1f;
+
+    // storage round trip
+    auto st = vtl::HipStorage<float>::from_cpu(x);
+    CHECK(st.count == x.size() && st.size == x.size() * 4);
+    CHECK(st.to_array() == x);
+    st.release();
+    CHECK(st.ptr == nullptr);
+
+    // quantize / dequantize vs oracle
+    auto xt = vtl::HipTensor<float>::from_host(x, {M, K});
+    CHECK(xt.is_matrix() && xt.strides == (std::vector<int>{K, 1}) && xt.numel() == (size_t)M * K);
+    for (int axis : {0, -1}) {
+        auto qs = vtl::quantize_i8(xt, axis);
+        std::vector<int8_t> qr(x.size());
+        std::vector<float> sr(axis == 0 ? M : 1);
+        vtl_ref_quantize_f32_i8(x.data(), M, K, axis == 0, qr.data(), sr.data());
+        CHECK(qs.first.cpu() == qr);
+        CHECK(qs.second.cpu() == sr);
+        auto d = vtl::dequantize(qs.first, qs.second, axis);
+        std::vector<float> dr(x.size());
+        vtl_ref_dequantize_i8_f32(qr.data(), sr.data(), M, K, axis == 0, dr.data());
+        CHECK(d.cpu() == dr);
+    }
+
+    // int8 gemm vs oracle
+    {
+        std::vector<int8_t> a((size_t)M * K), bt((size_t)N * K);
+        std::uniform_int_distribution<int> ud(-127, 127);
+        for (auto &v : a) v = (int8_t)ud(rng);
+        for (auto &v : bt) v = (int8_t)ud(rng);
+        auto A = vtl::HipTensor<int8_t>::from_host(a, {M, K});
+        auto B = vtl::HipTensor<int8_t>::from_host(bt, {N, K});
+        vtl::HipTensor<int32_t> C({M, N});
+        vtl::gemm_i8_hip(C, A, B);
+        std::vector<int32_t> ref((size_t)M * N);
+        vtl_ref_gemm_i8_i32(a.data(), bt.data(), ref.data(), M, N, K, 1);
+        CHECK(C.cpu() == ref);
+        vtl::HipTensor<int32_t> wrong({M, N + 1});
+        try {
+            vtl::gemm_i8_hip(wrong, A, B);
+            CHECK(false);
+        } catch (const std::invalid_argument &) {
+        }
+    }
+
+    // the Linear hook vs oracle (per-output-channel weights, per-token activations)
+    {
+        auto y = vtl::linear_forward_hip_f32(x, M, K, w, N, &b, true);
+        std::vector<int8_t> wq(w.size());
+        std::vector<float> sw(N), ref((size_t)M * N);
+        vtl_ref_quantize_f32_i8(w.data(), N, K, 1, wq.data(), sw.data());
+        vtl_ref_linear_f32_dynquant(x.data(), wq.data(), sw.data(), b.data(), ref.data(), M, N, K, 1, 1);
+        CHECK(y == ref);
+        try {
+            vtl::linear_forward_hip_f32(x, M, K + 1, w, N, &b);
+            CHECK(false);
+        } catch (const std::invalid_argument &) {
+        }
+    }
+    std::printf(failures ? "host mirror: %d failure(s)\n" : "host mirror: ok\n", failures);
+    return failures ? 1 : 0;
+}

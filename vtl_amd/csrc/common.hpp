@@ -18,6 +18,9 @@ int record_hip_error(hipError_t e, const char *what);
 // Checks the launch that was just made.
 int check_launch(const char *kernel_name);
 
+// Streaming copy kernel (quant.hip); false when alignment or size do not qualify.
+bool launch_copy(void *dst, const void *src, size_t bytes, hipStream_t st);
+
 constexpr int kWave = 64;
 
 }  // namespace vtlhip

@@ -378,6 +378,16 @@ __global__ __launch_bounds__(256) void relu_kernel(float *__restrict__ x, int64_
     }
 }
 
+// Plain streaming copy, one 16-byte vector per lane; also the kernel of known
+// traffic that hardware byte counters are calibrated against.
+__global__ __launch_bounds__(256) void copy_kernel(const float4_t *__restrict__ src,
+                                                   float4_t *__restrict__ dst, int64_t nv)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < nv)
+        __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+}
+
 inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
 constexpr int64_t kMaxGridX = 2147483647LL;
@@ -404,6 +414,21 @@ int launch_fill_zero(float *p, int64_t n, hipStream_t st)
 }  // namespace
 
 namespace vtlhip {
+
+// Device-to-device copy with the library's own kernel (16-byte aligned, size a
+// multiple of 16); returns false when the shape does not qualify.
+bool launch_copy(void *dst, const void *src, size_t bytes, hipStream_t st)
+{
+    if (!aligned(dst, 16) || !aligned(src, 16) || (bytes & 15))
+        return false;
+    const int64_t nv = (int64_t)(bytes >> 4);
+    const int64_t blocks = (nv + 255) / 256;
+    if (blocks > kMaxGridX)
+        return false;
+    hipLaunchKernelGGL(copy_kernel, dim3((unsigned)blocks), dim3(256), 0, st,
+                       reinterpret_cast<const float4_t *>(src), reinterpret_cast<float4_t *>(dst), nv);
+    return true;
+}
 
 // Per-row fused quantize; used by the C entry point and by the dynamic-quant
 // linear.  Preconditions were checked by the caller.

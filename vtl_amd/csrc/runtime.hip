@@ -124,6 +124,8 @@ int vtl_hip_memcpy_d2d(void *dst_device, const void *src_device, size_t bytes)
         return VTL_HIP_OK;
     if (!dst_device || !src_device)
         return VTL_HIP_ERR_INVALID_ARG;
+    if (launch_copy(dst_device, src_device, bytes, current_stream()))
+        return check_launch("copy_kernel");
     VTL_HIP_TRY(hipMemcpyAsync(dst_device, src_device, bytes, hipMemcpyDeviceToDevice, current_stream()));
     return VTL_HIP_OK;
 }

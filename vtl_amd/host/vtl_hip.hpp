@@ -1,0 +1,236 @@
+// C++ host-side mirror of the V binding of libvtlhip.so: HipStorage<T>,
+// HipTensor<T> and the Linear hook, written against the C ABI only
+// (include/vtl_hip.h; no HIP headers, no device code).  The reference's host
+// language is V, a compiled language with no toolchain here; this header plays
+// the role of storage/hip_d_hip.v, tensor_hip_d_hip.v and
+// nn/layers/linear_hip_d_hip.v for C++ callers and for the test program.
+//
+// Error behaviour follows the reference's GPU call sites
+// (storage/cuda_d_cuda.v:39-42,74-77): a non-zero status becomes an error
+// (here: vtl::HipError), never an abort, and there is no CPU fallback in here.
+#pragma once
+
+#include <cstdint>
+#include <cstdlib>
+#include <stdexcept>
+#include <string>
+#include <type_traits>
+#include <utility>
+#include <vector>
+
+#include "vtl_hip.h"
+
+namespace vtl {
+
+struct HipError : std::runtime_error {
+    int status;
+    HipError(const std::string &what, int st)
+        : std::runtime_error(what + " failed with status " + std::to_string(st) + ": " + vtl_hip_strerror(st)),
+          status(st) {}
+};
+
+inline void hip_check(int status, const char *what)
+{
+    if (status != VTL_HIP_OK)
+        throw HipError(what, status);
+}
+
+// `@[params] HipParams{device_id int = 0}` (cf. CudaParams, storage/cuda_d_cuda.v:9-11)
+struct HipParams {
+    int device_id = 0;
+};
+
+// `HipStorage[T]{ptr voidptr; size int; count int; device_id int}`
+// (cf. CudaStorage, storage/cuda_d_cuda.v:19-107).  Move-only; release() is
+// explicit as in the reference, the destructor is a safety net.
+template <typename T>
+class HipStorage {
+public:
+    void *ptr = nullptr;
+    size_t size = 0;   // bytes
+    size_t count = 0;  // elements
+    int device_id = 0;
+
+    HipStorage() = default;
+    HipStorage(size_t n, HipParams p = {}) : size(n * sizeof(T)), count(n), device_id(p.device_id)
+    {
+        hip_check(vtl_hip_set_device(p.device_id), "HipStorage: vtl_hip_set_device");
+        if (size)
+            hip_check(vtl_hip_malloc(&ptr, size), "HipStorage: vtl_hip_malloc");
+    }
+    // `(cpu &CpuStorage[T]) hip(params)`: allocate and copy, blocking
+    static HipStorage from_cpu(const std::vector<T> &host, HipParams p = {})
+    {
+        HipStorage s(host.size(), p);
+        if (s.size)
+            hip_check(vtl_hip_memcpy_h2d(s.ptr, host.data(), s.size), "HipStorage.hip: vtl_hip_memcpy_h2d");
+        return s;
+    }
+    HipStorage(const HipStorage &) = delete;
+    HipStorage &operator=(const HipStorage &) = delete;
+    HipStorage(HipStorage &&o) noexcept { *this = std::move(o); }
+    HipStorage &operator=(HipStorage &&o) noexcept
+    {
+        if (this != &o) {
+            release();
+            ptr = o.ptr; size = o.size; count = o.count; device_id = o.device_id;
+            o.ptr = nullptr; o.size = 0; o.count = 0;
+        }
+        return *this;
+    }
+    ~HipStorage() { release(); }
+
+    // `.to_array() ![]T`
+    std::vector<T> to_array() const
+    {
+        if (count && !ptr)
+            throw HipError("HipStorage.to_array: null pointer", VTL_HIP_ERR_INVALID_ARG);
+        std::vector<T> out(count);
+        if (size)
+            hip_check(vtl_hip_memcpy_d2h(out.data(), ptr, size), "HipStorage.to_array: vtl_hip_memcpy_d2h");
+        return out;
+    }
+    std::vector<T> cpu() const { return to_array(); }
+    void release() noexcept
+    {
+        if (ptr) {
+            vtl_hip_free(ptr);
+            ptr = nullptr;
+        }
+    }
+};
+
+// `HipTensor[T]{data; memory; size; shape; strides}` (cf. CudaTensor,
+// tensor_cuda_d_cuda.v:13-60), row-major only.
+template <typename T>
+class HipTensor {
+public:
+    HipStorage<T> data;
+    std::vector<int> shape;
+    std::vector<int> strides;
+    size_t size = 0;
+
+    HipTensor() = default;
+    HipTensor(std::vector<int> shp, HipParams p = {}) : shape(std::move(shp))
+    {
+        init_strides();
+        data = HipStorage<T>(size, p);
+    }
+    // `(t &Tensor[T]) hip(params)`
+    static HipTensor from_host(const std::vector<T> &host, std::vector<int> shp, HipParams p = {})
+    {
+        HipTensor t;
+        t.shape = std::move(shp);
+        t.init_strides();
+        if (t.size != host.size())
+            throw std::invalid_argument("HipTensor: shape does not match the number of elements");
+        t.data = HipStorage<T>::from_cpu(host, p);
+        return t;
+    }
+    std::vector<T> cpu() const { return data.to_array(); }
+    void release() { data.release(); }
+    int rank() const { return (int)shape.size(); }
+    size_t numel() const { return size; }
+    bool is_matrix() const { return rank() == 2; }
+    bool is_vector() const { return rank() == 1; }
+    bool is_square_matrix() const { return rank() == 2 && shape[0] == shape[1]; }
+
+private:
+    void init_strides()
+    {
+        size = 1;
+        strides.assign(shape.size(), 1);
+        for (int i = (int)shape.size() - 1; i >= 0; i--) {
+            strides[i] = (int)size;
+            size *= (size_t)shape[i];
+        }
+    }
+};
+
+inline int per_row_of(int axis)
+{
+    if (axis == -1)
+        return 0;
+    if (axis == 0)
+        return 1;
+    throw std::invalid_argument("axis: use -1 (whole tensor) or 0 (one scale per row)");
+}
+
+inline void matmul_shapes(const std::vector<int> &a, const std::vector<int> &bt, int &m, int &n, int &k)
+{
+    if (a.size() != 2 || bt.size() != 2)
+        throw std::invalid_argument("Matrix expected");
+    if (a[1] != bt[1])  // la.matmul, la/la.v:41-43
+        throw std::invalid_argument("Invalid shapes for matrix multiplication");
+    m = a[0]; n = bt[0]; k = a[1];
+}
+
+// `quantize_i8(axis) !(&HipTensor[i8], &HipTensor[f32])`
+inline std::pair<HipTensor<int8_t>, HipTensor<float>> quantize_i8(const HipTensor<float> &x, int axis)
+{
+    if (!x.is_matrix())
+        throw std::invalid_argument("Matrix expected");
+    const int per_row = per_row_of(axis);
+    HipParams p{x.data.device_id};
+    HipTensor<int8_t> q({x.shape[0], x.shape[1]}, p);
+    HipTensor<float> s({per_row ? x.shape[0] : 1}, p);
+    hip_check(vtl_hip_quantize_f32_i8((const float *)x.data.ptr, x.shape[0], x.shape[1], per_row,
+                                      (int8_t *)q.data.ptr, (float *)s.data.ptr),
+              "vtl_hip_quantize_f32_i8");
+    return {std::move(q), std::move(s)};
+}
+
+// `dequantize(scales, axis) !&HipTensor[f32]`
+inline HipTensor<float> dequantize(const HipTensor<int8_t> &q, const HipTensor<float> &scales, int axis)
+{
+    if (!q.is_matrix())
+        throw std::invalid_argument("Matrix expected");
+    const int per_row = per_row_of(axis);
+    if (scales.size != (size_t)(per_row ? q.shape[0] : 1))
+        throw std::invalid_argument("dequantize: number of scales does not match");
+    HipTensor<float> x({q.shape[0], q.shape[1]}, HipParams{q.data.device_id});
+    hip_check(vtl_hip_dequantize_i8_f32((const int8_t *)q.data.ptr, (const float *)scales.data.ptr, q.shape[0],
+                                        q.shape[1], per_row, (float *)x.data.ptr),
+              "vtl_hip_dequantize_i8_f32");
+    return x;
+}
+
+// `gemm_i8_hip(dst, a, b) !`
+inline void gemm_i8_hip(HipTensor<int32_t> &dst, const HipTensor<int8_t> &a, const HipTensor<int8_t> &bt)
+{
+    int m, n, k;
+    matmul_shapes(a.shape, bt.shape, m, n, k);
+    if (dst.shape != std::vector<int>{m, n})
+        throw std::invalid_argument("gemm_i8_hip: dst shape");
+    hip_check(vtl_hip_gemm_i8_i32((const int8_t *)a.data.ptr, (const int8_t *)bt.data.ptr, (int32_t *)dst.data.ptr,
+                                  m, n, k),
+              "vtl_hip_gemm_i8_i32");
+}
+
+// `linear_forward_hip_f32(x, weights, bias) !&vtl.Tensor[f32]`: host tensors in,
+// host tensor out (every GPU path of the reference returns host tensors,
+// docs/DEVICE_MEMORY.md:9-16).  weights are [out, in] as stored, bias [1, out].
+inline std::vector<float> linear_forward_hip_f32(const std::vector<float> &x, int m, int k,
+                                                 const std::vector<float> &weights, int n,
+                                                 const std::vector<float> *bias, bool relu = false)
+{
+    if (x.size() != (size_t)m * k || weights.size() != (size_t)n * k)
+        throw std::invalid_argument("Invalid shapes for matrix multiplication");
+    if (bias && bias->size() != (size_t)n)
+        throw std::invalid_argument("bias: one entry per output feature expected");
+    auto w_dev = HipTensor<float>::from_host(weights, {n, k});
+    auto wq = quantize_i8(w_dev, 0);
+    auto x_dev = HipTensor<float>::from_host(x, {m, k});
+    HipStorage<float> b_dev;
+    if (bias)
+        b_dev = HipStorage<float>::from_cpu(*bias);
+    HipStorage<uint8_t> ws(vtl_hip_linear_f32_dynquant_workspace(m, k));
+    HipTensor<float> y({m, n});
+    hip_check(vtl_hip_linear_f32_dynquant((const float *)x_dev.data.ptr, (const int8_t *)wq.first.data.ptr,
+                                          (const float *)wq.second.data.ptr, (const float *)b_dev.ptr,
+                                          (float *)y.data.ptr, m, n, k, relu ? 1 : 0, ws.ptr, ws.size),
+              "vtl_hip_linear_f32_dynquant");
+    return y.cpu();
+}
+
+}  // namespace vtl
