@@ -168,6 +168,85 @@ def bench_quant(timer: Timer, steps: int, warmup: int, cpu: bool):
     return out
 
 
+def bench_other_configs(timer: Timer, steps: int, warmup: int):
+    """Timings of the remaining configurations (parity for them is in tests/):
+    configs[0] MNIST-MLP first layer, configs[3] decode-shaped linear with
+    per-token quantization on the fly, configs[4] 3-layer int8 MLP chain."""
+    from vtl_amd.storage import HipStorage
+    out = {}
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        _, dev_ms = timer.run(fn, steps)
+        return dev_ms / steps * 1e3   # microseconds
+
+    # configs[0]: per-tensor quantize of x, int8 linear (weights quantized once, untimed)
+    x, w, b = workloads.mnist_mlp_first_layer()
+    X, W, B = HipTensor.from_host(x), HipTensor.from_host(w), HipTensor.from_host(b.reshape(-1))
+    Wq, Sw = W.quantize_i8(-1)
+    Xq, Sx = HipTensor.empty([64, 784], np.int8), HipTensor.empty([1], np.float32)
+    Y = HipTensor.empty([64, 256], np.float32)
+
+    def c1():
+        capi.call("vtl_hip_quantize_f32_i8", X.ptr, 64, 784, 0, Xq.ptr, Sx.ptr)
+        capi.call("vtl_hip_linear_i8_f32", Xq.ptr, Sx.ptr, 0, Wq.ptr, Sw.ptr, 0, B.ptr, Y.ptr, 64, 256, 784, 0)
+    out["configs[0] mnist first layer [64,784]x[256,784]^T"] = {"us": timed(c1), "ops": 2.0 * 64 * 784 * 256}
+    for h in (X, W, B, Wq, Sw, Xq, Sx, Y):
+        h.release()
+
+    # configs[3]: K=4096, N=14336, M in {1,8,32,128}
+    k, n = 4096, 14336
+    rng = np.random.Generator(np.random.Philox(3))
+    Wq = HipTensor.from_host(rng.integers(-127, 128, (n, k), dtype=np.int8))
+    Sw = HipTensor.from_host((rng.uniform(0.5, 1.5, n) * 1e-3).astype(np.float32))
+    dec = {}
+    for m in (1, 8, 32, 128):
+        X = HipTensor.from_host(rng.standard_normal((m, k), dtype=np.float32))
+        Y = HipTensor.empty([m, n], np.float32)
+        need = int(capi.lib().vtl_hip_linear_f32_dynquant_workspace(m, k))
+        ws = HipStorage.empty(need, np.uint8)
+
+        def c4():
+            capi.call("vtl_hip_linear_f32_dynquant", X.ptr, Wq.ptr, Sw.ptr, None, Y.ptr, m, n, k, 0, ws.ptr, ws.size)
+        us = timed(c4)
+        algo = n * k + 16384.0 * m + 57344.0 * m + 57344.0     # Wq + X f32 + Y f32 + sw
+        dec[f"M={m}"] = {"us": us, "GB/s": algo / us / 1e3, "frac_of_hbm_peak": algo / us / 1e3 / PEAK_HBM_GBPS,
+                         "TOPS": 2.0 * m * n * k / us / 1e6, "algorithmic_bytes": algo}
+        capi.call("vtl_hip_sync")
+        for h in (X, Y):
+            h.release()
+        ws.release()
+    out["configs[3] decode linear K=4096 N=14336 (quantize on the fly + int8 linear)"] = dec
+    Wq.release()
+    Sw.release()
+
+    # configs[4]: 256x4096 -> 11008 -> ReLU -> 4096 -> ReLU -> 1024, device-resident chain
+    dims, m = (4096, 11008, 4096, 1024), 256
+    Ws = [HipTensor.from_host(rng.integers(-127, 128, (dims[i + 1], dims[i]), dtype=np.int8)) for i in range(3)]
+    Ss = [HipTensor.from_host((rng.uniform(0.5, 1.5, dims[i + 1]) * 1e-3).astype(np.float32)) for i in range(3)]
+    X = HipTensor.from_host(rng.standard_normal((m, dims[0]), dtype=np.float32))
+    Ys = [HipTensor.empty([m, dims[i + 1]], np.float32) for i in range(3)]
+    ws = HipStorage.empty(int(capi.lib().vtl_hip_linear_f32_dynquant_workspace(m, max(dims))), np.uint8)
+
+    def c5():
+        cur = X
+        for i in range(3):
+            capi.call("vtl_hip_linear_f32_dynquant", cur.ptr, Ws[i].ptr, Ss[i].ptr, None, Ys[i].ptr, m,
+                      dims[i + 1], dims[i], 1 if i < 2 else 0, ws.ptr, ws.size)
+            cur = Ys[i]
+    us = timed(c5)
+    ops = 2.0 * m * sum(dims[i] * dims[i + 1] for i in range(3))
+    wbytes = float(sum(dims[i] * dims[i + 1] for i in range(3)))
+    out["configs[4] int8 MLP chain 256x4096->11008->4096->1024"] = {
+        "us": us, "TOPS": ops / us / 1e6, "weight_GB/s": wbytes / us / 1e3, "ops": ops}
+    capi.call("vtl_hip_sync")
+    for h in Ws + Ss + Ys + [X]:
+        h.release()
+    ws.release()
+    return out
+
+
 def bench_copy_calibration(timer: Timer, steps: int, warmup: int):
     """Plain device-to-device copy of 1 GiB with the library's copy kernel: the
     kernel of known traffic (1 GiB read + 1 GiB written per launch) that the
@@ -242,6 +321,8 @@ def main() -> int:
     if qd:
         line["quantize"] = qd["quantize"]
         line["dequantize"] = qd["dequantize"]
+    if args.only == "all":
+        line["other_configs"] = bench_other_configs(timer, args.steps, args.warmup)
     print(json.dumps(line))
     return 0
 

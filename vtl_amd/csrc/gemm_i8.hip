@@ -7,6 +7,9 @@
 // are "rows of K bytes" and a lane's MFMA operand is 16 consecutive K bytes of
 // one row.  Integer accumulation is order-free, so the only requirement on the
 // K order inside the instruction is that A and B use the same one.
+#include <stdio.h>
+#include <stdlib.h>
+
 #include "common.hpp"
 
 using namespace vtlhip;
@@ -36,6 +39,8 @@ struct GemmArgs {
     int sa_stride;  // 1: one scale per row of A, 0: one scale
     int sw_stride;  // 1: one scale per row of Bt, 0: one scale
     int relu;
+    int splits;         // K is cut into this many ranges, one workgroup each (1 = no split)
+    int32_t *partials;  // [splits][M][N] int32 partial sums when splits > 1
 };
 
 // LDS tiles are rows of BK bytes (BK/16 chunks of 16 bytes).  The chunk index
@@ -63,10 +68,10 @@ __device__ __forceinline__ void wait_vmcnt()
 // Workgroups are dealt round-robin to the 8 XCDs; renumber them so that each
 // XCD (own L2) works on a compact patch of the tile grid, then walk the grid
 // in groups of 8 tile rows.
-__device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int &tile_m, int &tile_n)
+__device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int block, int &tile_m, int &tile_n)
 {
     const int total = tiles_m * tiles_n;
-    int pid = blockIdx.x;
+    int pid = block;
     if ((total & 7) == 0)
         pid = (pid & 7) * (total >> 3) + (pid >> 3);
     constexpr int GM = 8;
@@ -148,6 +153,9 @@ __device__ __forceinline__ void epilogue(v16i (&acc)[WM / 32][WN / 32], const Ge
                             y = 0.0f;
                         reinterpret_cast<float *>(g.out)[(int64_t)m * N + n] = y;
                     }
+                    // keep the compiler from hoisting every scale read of the tile to the
+                    // top of the epilogue, which costs more registers than there are
+                    asm volatile("" ::: "memory");
                 }
             }
         }
@@ -163,7 +171,7 @@ __device__ __forceinline__ void epilogue(v16i (&acc)[WM / 32][WN / 32], const Ge
 // and the first operand reads of the next tile hide behind that step's MFMAs.
 // Requires K % BK == 0; with EDGE, rows past M / N are clamped on load and
 // masked on store.
-template <int BM, int BN, int BK, int NSTAGE, int WR, int WC, bool F32OUT, bool EDGE>
+template <int BM, int BN, int BK, int NSTAGE, int WR, int WC, bool F32OUT, bool EDGE, bool SPLIT>
 __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArgs g)
 {
     constexpr int NW = WR * WC, NT = 64 * NW;
@@ -180,11 +188,18 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArg
 
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int M = g.M, N = g.N, K = g.K;
+    // block -> (output tile, K range): consecutive blocks are the K ranges of one tile
+    const int nsplit = SPLIT ? g.splits : 1;
+    const int split = SPLIT ? (int)(blockIdx.x % nsplit) : 0;
     int tile_m, tile_n;
-    tile_of_block((M + BM - 1) / BM, (N + BN - 1) / BN, tile_m, tile_n);
+    tile_of_block((M + BM - 1) / BM, (N + BN - 1) / BN, SPLIT ? (int)(blockIdx.x / nsplit) : (int)blockIdx.x,
+                  tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int wr = w / WC, wc = w % WC;
+    const int kt_all = K / BK;
+    const int kt_begin = SPLIT ? (int)((int64_t)kt_all * split / nsplit) : 0;
+    const int kt_end = SPLIT ? (int)((int64_t)kt_all * (split + 1) / nsplit) : kt_all;
 
     // ---- global -> LDS ----
     const int lrow = RPI * w + lane / CPR;                  // tile row of this lane for j = 0
@@ -206,7 +221,7 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArg
     auto issue = [&](int kt, int st) {
         char *sa_ = smem + st * STAGE;
         char *sb_ = sa_ + BM * BK;
-        const int64_t ko = (int64_t)kt * BK;
+        const int64_t ko = (int64_t)(kt_begin + kt) * BK;
 #pragma unroll
         for (int j = 0; j < A_PW; j++)
             __builtin_amdgcn_global_load_lds(VTL_GPTR(EDGE ? pa[EDGE ? j : 0] + ko : pa[0] + ko + j * jstride),
@@ -264,7 +279,7 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArg
         }
     };
 
-    const int KT = K / BK;
+    const int KT = kt_end - kt_begin;
 #pragma unroll
     for (int st = 0; st < NSTAGE; st++)
         if (st < KT)
@@ -307,7 +322,40 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArg
     }
     mma((KS - 1) & 1);
 
-    epilogue<BM, BN, WM, WN, F32OUT, EDGE, NT>(acc, g, m0, n0, wr, wc, smem);
+    if constexpr (SPLIT) {
+        // raw partial sums of this K range; splitk_finalize_kernel adds the ranges up
+        GemmArgs gp = g;
+        gp.out = g.partials + (int64_t)split * M * N;
+        epilogue<BM, BN, WM, WN, false, EDGE, NT>(acc, gp, m0, n0, wr, wc, smem);
+    } else {
+        epilogue<BM, BN, WM, WN, F32OUT, EDGE, NT>(acc, g, m0, n0, wr, wc, smem);
+    }
+}
+
+// Sums the int32 partial results of a split-K launch (exact, order-free) and
+// applies the epilogue.  One thread per output element, n fastest.
+template <bool F32OUT>
+__global__ __launch_bounds__(256) void splitk_finalize_kernel(const GemmArgs g)
+{
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t mn = (int64_t)g.M * g.N;
+    if (idx >= mn)
+        return;
+    int acc = 0;
+    for (int s = 0; s < g.splits; s++)
+        acc += g.partials[(int64_t)s * mn + idx];
+    if (F32OUT) {
+        const int m = (int)(idx / g.N), n = (int)(idx % g.N);
+        const float sc = g.sa[(int64_t)m * g.sa_stride] * g.sw[(int64_t)n * g.sw_stride];
+        float y = (float)acc * sc;
+        if (g.bias)
+            y = y + g.bias[n];
+        if (g.relu && y < 0.0f)
+            y = 0.0f;
+        reinterpret_cast<float *>(g.out)[idx] = y;
+    } else {
+        reinterpret_cast<int32_t *>(g.out)[idx] = acc;
+    }
 }
 
 // Register-staged tile kernel for K that is a multiple of 16 but not of the
@@ -330,7 +378,7 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_tile_kernel(const GemmAr
 
     const int M = g.M, N = g.N, K = g.K;
     int tile_m, tile_n;
-    tile_of_block((M + BM - 1) / BM, (N + BN - 1) / BN, tile_m, tile_n);
+    tile_of_block((M + BM - 1) / BM, (N + BN - 1) / BN, (int)blockIdx.x, tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wr = wave / WC, wc = wave % WC;
@@ -455,18 +503,69 @@ int launch_with_lds(Kern kern, bool &attr_done, int lds, int tiles, int threads,
     return check_launch(name);
 }
 
+// Scratch for split-K partial sums, owned by the library, grown on demand and
+// kept until the process ends (one host thread per device).
+int32_t *splitk_workspace(size_t bytes)
+{
+    static int32_t *buf = nullptr;
+    static size_t cap = 0;
+    if (bytes > cap) {
+        if (buf) {
+            (void)hipStreamSynchronize(current_stream());
+            (void)hipFree(buf);
+            buf = nullptr;
+            cap = 0;
+        }
+        const size_t want = bytes < (size_t(32) << 20) ? (size_t(32) << 20) : bytes;
+        if (hipMalloc(reinterpret_cast<void **>(&buf), want) != hipSuccess) {
+            (void)hipGetLastError();
+            buf = nullptr;
+            return nullptr;
+        }
+        cap = want;
+    }
+    return buf;
+}
+
 template <int BM, int BN, int BK, int NSTAGE, int WR, int WC, bool F32OUT>
-int launch_dma(const GemmArgs &g, hipStream_t st)
+int launch_dma(GemmArgs g, int splits, hipStream_t st)
 {
     constexpr int lds = NSTAGE * (BM + BN) * BK;
     static_assert(lds >= (BM + 2 * BN) * 4, "epilogue staging fits in the operand buffers");
+    static_assert((NSTAGE - 1) * ((BM + BN) / (64 / (BK / 16)) / (WR * WC)) <= 63, "vmcnt is a 6-bit counter");
     const int tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
-    static bool done_edge = false, done_full = false;
-    if ((g.M % BM) || (g.N % BN))
-        return launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, F32OUT, true>, done_edge, lds,
-                               tiles, 64 * WR * WC, g, st, "gemm_i8_dma_kernel");
-    return launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, F32OUT, false>, done_full, lds,
-                           tiles, 64 * WR * WC, g, st, "gemm_i8_dma_kernel");
+    const int kt_all = g.K / BK;
+    if (splits > kt_all)
+        splits = kt_all;
+    if (splits < 1)
+        splits = 1;
+    g.splits = splits;
+    if (splits > 1) {
+        g.partials = splitk_workspace((size_t)splits * (size_t)g.M * (size_t)g.N * sizeof(int32_t));
+        if (!g.partials)
+            return VTL_HIP_ERR_OUT_OF_MEMORY;
+    }
+    static bool done[4] = {false, false, false, false};
+    const bool edge = (g.M % BM) || (g.N % BN);
+    int rc;
+    // the partial sums of a split launch are int32 whatever the final type is
+    if (splits > 1 && edge)
+        rc = launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, false, true, true>, done[0], lds,
+                             tiles * splits, 64 * WR * WC, g, st, "gemm_i8_dma_kernel");
+    else if (splits > 1)
+        rc = launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, false, false, true>, done[1], lds,
+                             tiles * splits, 64 * WR * WC, g, st, "gemm_i8_dma_kernel");
+    else if (edge)
+        rc = launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, F32OUT, true, false>, done[2], lds,
+                             tiles, 64 * WR * WC, g, st, "gemm_i8_dma_kernel");
+    else
+        rc = launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, F32OUT, false, false>, done[3], lds,
+                             tiles, 64 * WR * WC, g, st, "gemm_i8_dma_kernel");
+    if (rc != VTL_HIP_OK || splits == 1)
+        return rc;
+    const int64_t blocks = ((int64_t)g.M * g.N + 255) / 256;
+    hipLaunchKernelGGL((splitk_finalize_kernel<F32OUT>), dim3((unsigned)blocks), dim3(256), 0, st, g);
+    return check_launch("splitk_finalize_kernel");
 }
 
 template <int BM, int BN, int WR, int WC, bool F32OUT>
@@ -479,6 +578,64 @@ int launch_tile(const GemmArgs &g, hipStream_t st)
                            "gemm_i8_tile_kernel");
 }
 
+// The DMA-kernel instantiations, smallest tile first.
+struct TileConfig {
+    int bm, bn;
+    float step_cycles;  // one 128-byte K step of one workgroup: max(MFMA time, L2->LDS fill at ~40 B/clk)
+    int wgs_per_cu;     // workgroups that fit a compute unit's LDS together
+};
+constexpr TileConfig kTileConfigs[] = {
+    {32, 64, 330.f, 1}, {32, 128, 520.f, 2}, {64, 128, 560.f, 2}, {128, 128, 830.f, 2}, {256, 256, 2600.f, 1}};
+constexpr int kNumTileConfigs = 5;
+
+template <bool F32OUT>
+int launch_config(int idx, const GemmArgs &g, int splits, hipStream_t st)
+{
+    switch (idx) {
+    case 0: return launch_dma<32, 64, 128, 8, 1, 2, F32OUT>(g, splits, st);
+    case 1: return launch_dma<32, 128, 128, 4, 1, 4, F32OUT>(g, splits, st);
+    case 2: return launch_dma<64, 128, 128, 3, 2, 2, F32OUT>(g, splits, st);
+    case 3: return launch_dma<128, 128, 128, 2, 2, 2, F32OUT>(g, splits, st);
+    default: return launch_dma<256, 256, 128, 2, 2, 4, F32OUT>(g, splits, st);
+    }
+}
+
+// Picks the tile and the number of K ranges that minimise a simple cost
+// model, the larger of
+//   latency:    rounds of workgroups over the resident slots x K steps per workgroup x step cost
+//   throughput: all K steps of all workgroups x step cost / 256 compute units
+// plus, for split K, the extra launch and the pass over the partial sums.
+// The constants were fitted to measured times of the benchmark shapes.
+void choose_config(int M, int N, int K, int &best_idx, int &best_splits)
+{
+    const int kt_all = K / 128;
+    float best = 3.0e38f;
+    best_idx = kNumTileConfigs - 1;
+    best_splits = 1;
+    for (int i = 0; i < kNumTileConfigs; i++) {
+        const TileConfig &c = kTileConfigs[i];
+        if (i > 0 && kTileConfigs[i - 1].bm >= M && c.bm > kTileConfigs[i - 1].bm)
+            break;  // a taller tile would only add padding rows
+        const int64_t tiles = (int64_t)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
+        for (int s = 1; s <= 16; s *= 2) {
+            if (s > 1 && kt_all / s < 4)
+                break;
+            const int64_t rounds = (tiles * s + 256 * c.wgs_per_cu - 1) / (256 * c.wgs_per_cu);
+            const int steps = (kt_all + s - 1) / s;
+            const float latency = (float)rounds * ((float)steps * c.step_cycles + 3000.f);
+            const float throughput = (float)tiles * (float)s * (float)steps * c.step_cycles / 256.f + 3000.f;
+            float cost = latency > throughput ? latency : throughput;
+            if (s > 1)
+                cost += 6000.f + (float)s * (float)M * (float)N * 4.0f / 2500.f;
+            if (cost < best) {
+                best = cost;
+                best_idx = i;
+                best_splits = s;
+            }
+        }
+    }
+}
+
 template <bool F32OUT>
 int launch_gemm(const GemmArgs &g, hipStream_t st)
 {
@@ -489,18 +646,19 @@ int launch_gemm(const GemmArgs &g, hipStream_t st)
         hipLaunchKernelGGL((gemm_i8_naive_kernel<F32OUT>), grid, dim3(256), 0, st, g);
         return check_launch("gemm_i8_naive_kernel");
     }
-    const int64_t t256 = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256);
-    const int64_t t128 = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
     if (g.K % 128 == 0) {
-        // Largest tile that still gives most compute units a workgroup.
-        if (g.M > 128 && t256 >= 200)
-            return launch_dma<256, 256, 128, 2, 2, 4, F32OUT>(g, st);
-        if (g.M > 64)
-            return launch_dma<128, 128, 128, 2, 2, 2, F32OUT>(g, st);
-        if (g.M > 32)
-            return launch_dma<64, 128, 128, 2, 2, 2, F32OUT>(g, st);
-        return launch_dma<32, 128, 128, 2, 1, 4, F32OUT>(g, st);
+        int idx, splits;
+        choose_config(g.M, g.N, g.K, idx, splits);
+        if (const char *force = getenv("VTL_HIP_GEMM_CONFIG")) {  // tuning knob: "<tile index>,<splits>"
+            int fi = -1, fs = 1;
+            if (sscanf(force, "%d,%d", &fi, &fs) >= 1 && fi >= 0 && fi < kNumTileConfigs) {
+                idx = fi;
+                splits = fs;
+            }
+        }
+        return launch_config<F32OUT>(idx, g, splits, st);
     }
+    const int64_t t128 = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
     if (g.M > 64 && t128 >= 64)
         return launch_tile<128, 128, 2, 2, F32OUT>(g, st);
     if (g.M > 32)
@@ -530,7 +688,7 @@ int vtl_hip_gemm_i8_i32(const int8_t *A, const int8_t *Bt, int32_t *C, int M, in
         return VTL_HIP_OK;
     if (K == 0)
         return VTL_HIP_ERR_UNSUPPORTED;  // la.matmul has no empty inner dimension either
-    GemmArgs g{A, Bt, C, nullptr, nullptr, nullptr, M, N, K, 0, 0, 0};
+    GemmArgs g{A, Bt, C, nullptr, nullptr, nullptr, M, N, K, 0, 0, 0, 1, nullptr};
     return launch_gemm<false>(g, current_stream());
 }
 
@@ -547,7 +705,7 @@ int vtl_hip_linear_i8_f32(const int8_t *A, const float *sa, int sa_per_row, cons
         return VTL_HIP_OK;
     if (K == 0)
         return VTL_HIP_ERR_UNSUPPORTED;  // la.matmul rejects empty inner dimensions as well
-    GemmArgs g{A, Wq, Y, sa, sw, bias, M, N, K, sa_per_row ? 1 : 0, sw_per_col ? 1 : 0, relu ? 1 : 0};
+    GemmArgs g{A, Wq, Y, sa, sw, bias, M, N, K, sa_per_row ? 1 : 0, sw_per_col ? 1 : 0, relu ? 1 : 0, 1, nullptr};
     return launch_gemm<true>(g, current_stream());
 }
 
@@ -582,7 +740,7 @@ int vtl_hip_linear_f32_dynquant(const float *X, const int8_t *Wq, const float *s
     st = launch_quantize_rows(X, M, K, xq, sx, current_stream());
     if (st != VTL_HIP_OK)
         return st;
-    GemmArgs g{xq, Wq, Y, sx, sw, bias, M, N, K, 1, 1, relu ? 1 : 0};
+    GemmArgs g{xq, Wq, Y, sx, sw, bias, M, N, K, 1, 1, relu ? 1 : 0, 1, nullptr};
     return launch_gemm<true>(g, current_stream());
 }
 
