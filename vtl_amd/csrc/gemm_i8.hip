@@ -358,6 +358,183 @@ __global__ __launch_bounds__(256) void splitk_finalize_kernel(const GemmArgs g)
     }
 }
 
+// Weight-streaming kernel for M <= 32 (decode-shaped linear): bound by reading
+// the weight matrix once, so the design goal is bytes in flight and long
+// contiguous reads, not MFMA rate.  A workgroup owns 32 weight rows (128 KiB of
+// contiguous memory when K = 4096); its NWAVE waves split K between them and
+// each wave runs a PRIVATE software pipeline - its own LDS ring of STAGES
+// slots (32 rows x 256 bytes of Wq plus the activation rows that exist),
+// filled by its own direct-to-LDS loads and released by its own vmcnt waits -
+// so there is no workgroup barrier in the K loop at all.  Reads are 256 bytes
+// per row per step: measured, 128-byte pieces at row stride reach 5.4 TB/s on
+// this matrix, 256-byte pieces 7.8 TB/s.  The waves' int32 partial tiles are
+// added up through LDS at the end (exact), then the f32 epilogue runs.
+// MFMA operand A = weight rows (n), operand B = activation rows (m), so a
+// lane ends up with four consecutive n of one m: 16-byte stores along Y rows.
+// Only the 8*XJ activation rows that can exist (M <= 8*XJ) are loaded; lanes
+// of absent rows re-read existing ones and their output columns are never
+// stored.  Requires K % 256 == 0; rows past N are clamped on load and masked
+// on store.
+template <int NWAVE, int STAGES, int XJ, bool F32OUT>
+__global__ __launch_bounds__(64 * NWAVE) void linear_skinny_kernel(const GemmArgs g)
+{
+    constexpr int BK = 256;
+    constexpr int WCHUNK = 32 * BK;              // 8 KiB of weights per slot
+    constexpr int XROWS = 8 * XJ;
+    constexpr int SLOT = WCHUNK + XROWS * BK;
+    constexpr int WLOADS = 8, XLOADS = 2 * XJ;   // wave instructions (4 rows x 256 bytes each)
+    constexpr int LOADS = WLOADS + XLOADS;
+    constexpr int KS = BK / 32;                  // MFMA k-steps per slot
+    static_assert((STAGES - 1) * LOADS <= 63, "vmcnt is a 6-bit counter");
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int M = g.M, N = g.N, K = g.K;
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int n0 = blockIdx.x * 32;
+    char *ring = smem + w * (STAGES * SLOT);
+
+    // K range of this wave, in 256-byte chunks
+    const int kc_all = K / BK;
+    const int kc_begin = (int)((int64_t)kc_all * w / NWAVE);
+    const int kc_end = (int)((int64_t)kc_all * (w + 1) / NWAVE);
+    const int KC = kc_end - kc_begin;
+
+    // global -> LDS: instruction j covers tile rows 4j .. 4j+3, 16 lanes per 256-byte row;
+    // LDS rows are 256 bytes, 16-byte chunk index XOR (row & 15)
+    const int lrow = lane >> 4;
+    const int8_t *pw[WLOADS];
+    const int8_t *px[XLOADS];
+#pragma unroll
+    for (int j = 0; j < WLOADS; j++) {
+        const int row = lrow + 4 * j;
+        const int lc = (lane & 15) ^ (row & 15);
+        pw[j] = g.Bt + (int64_t)min(n0 + row, N - 1) * K + (int64_t)kc_begin * BK + lc * 16;
+    }
+#pragma unroll
+    for (int j = 0; j < XLOADS; j++) {
+        const int row = lrow + 4 * j;
+        const int lc = (lane & 15) ^ (row & 15);
+        px[j] = g.A + (int64_t)min(row, M - 1) * K + (int64_t)kc_begin * BK + lc * 16;
+    }
+    auto issue = [&](int c, int st) {
+        char *sw_ = ring + st * SLOT;
+        char *sx_ = sw_ + WCHUNK;
+        const int64_t ko = (int64_t)c * BK;
+#pragma unroll
+        for (int j = 0; j < WLOADS; j++)
+            __builtin_amdgcn_global_load_lds(VTL_GPTR(pw[j] + ko), VTL_LPTR(sw_ + j * 1024), 16, 0, 0);
+#pragma unroll
+        for (int j = 0; j < XLOADS; j++)
+            __builtin_amdgcn_global_load_lds(VTL_GPTR(px[j] + ko), VTL_LPTR(sx_ + j * 1024), 16, 0, 0);
+    };
+
+    v16i acc0, acc1;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        acc0[r] = 0;
+        acc1[r] = 0;
+    }
+    const int frow = lane & 31, fh = lane >> 5;
+    const int xrow = frow & (XROWS - 1);  // absent activation rows alias existing ones
+    int woff[KS], xoff[KS];
+#pragma unroll
+    for (int s = 0; s < KS; s++) {
+        woff[s] = frow * BK + ((((2 * s + fh) ^ frow) & 15) << 4);
+        xoff[s] = xrow * BK + ((((2 * s + fh) ^ xrow) & 15) << 4);
+    }
+
+#pragma unroll
+    for (int st = 0; st < STAGES - 1; st++)
+        if (st < KC)
+            issue(st, st);
+    int st_c = 0, st_l = STAGES - 1;
+    for (int c = 0; c < KC; c++) {
+        if (c + STAGES - 1 < KC) {
+            issue(c + STAGES - 1, st_l);
+            wait_vmcnt<(STAGES - 1) * LOADS>();  // chunk c has landed
+        } else {
+            wait_vmcnt<0>();
+        }
+        const char *sw_ = ring + st_c * SLOT;
+        const char *sx_ = sw_ + WCHUNK;
+        v4i wf[KS], xf[KS];
+#pragma unroll
+        for (int s = 0; s < KS; s++) {
+            wf[s] = *reinterpret_cast<const v4i *>(sw_ + woff[s]);
+            xf[s] = *reinterpret_cast<const v4i *>(sx_ + xoff[s]);
+        }
+#pragma unroll
+        for (int s = 0; s < KS; s += 2) {
+            acc0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[s], xf[s], acc0, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[s + 1], xf[s + 1], acc1, 0, 0, 0);
+        }
+        // the reads of this slot are complete before it is refilled in the next iteration
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        st_c = (st_c + 1 == STAGES) ? 0 : st_c + 1;
+        st_l = (st_l + 1 == STAGES) ? 0 : st_l + 1;
+    }
+
+    // ---- add the waves' partial tiles up through LDS: part[wave][m][n] ----
+    __syncthreads();  // every wave is done with its ring
+    int *part = reinterpret_cast<int *>(smem);
+    {
+        const int m = lane & 31, nb = (lane >> 5) * 4;
+#pragma unroll
+        for (int rq = 0; rq < 4; rq++) {
+            v4i v;
+#pragma unroll
+            for (int k = 0; k < 4; k++)
+                v[k] = acc0[rq * 4 + k] + acc1[rq * 4 + k];
+            *reinterpret_cast<v4i *>(part + w * 1024 + m * 32 + 8 * rq + nb) = v;
+        }
+    }
+    __syncthreads();
+    // 256 (m, 4 x n) items; 8 threads cover the 128-byte row segment of one m
+    for (int item = tid; item < 256; item += 64 * NWAVE) {
+        const int m = item >> 3, nq = (item & 7) * 4;
+        v4i sum = *reinterpret_cast<const v4i *>(part + m * 32 + nq);
+#pragma unroll
+        for (int ww = 1; ww < NWAVE; ww++)
+            sum += *reinterpret_cast<const v4i *>(part + ww * 1024 + m * 32 + nq);
+        if (m >= M)
+            continue;
+        const int n = n0 + nq;
+        const int64_t o = (int64_t)m * N + n;
+        if constexpr (F32OUT) {
+            const float a = g.sa[(int64_t)m * g.sa_stride];
+            float y[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                if (n + k < N) {
+                    const float sc = a * g.sw[(int64_t)(n + k) * g.sw_stride];
+                    float v = (float)sum[k] * sc;
+                    if (g.bias)
+                        v = v + g.bias[n + k];
+                    if (g.relu && v < 0.0f)
+                        v = 0.0f;
+                    y[k] = v;
+                }
+            }
+            if (n + 3 < N && (N & 3) == 0) {
+                *reinterpret_cast<f4 *>(reinterpret_cast<float *>(g.out) + o) = f4{y[0], y[1], y[2], y[3]};
+            } else {
+#pragma unroll
+                for (int k = 0; k < 4; k++)
+                    if (n + k < N)
+                        reinterpret_cast<float *>(g.out)[o + k] = y[k];
+            }
+        } else {
+            if (n + 3 < N && (N & 3) == 0) {
+                *reinterpret_cast<v4i *>(reinterpret_cast<int32_t *>(g.out) + o) = sum;
+            } else {
+#pragma unroll
+                for (int k = 0; k < 4; k++)
+                    if (n + k < N)
+                        reinterpret_cast<int32_t *>(g.out)[o + k] = sum[k];
+            }
+        }
+    }
+}
+
 // Register-staged tile kernel for K that is a multiple of 16 but not of the
 // DMA kernel's tile depth: global -> VGPR -> LDS, zero-filled K tail.
 template <int BM, int BN, int WR, int WC, bool F32OUT>
@@ -636,6 +813,30 @@ void choose_config(int M, int N, int K, int &best_idx, int &best_splits)
     }
 }
 
+template <int NWAVE, int STAGES, int XJ, bool F32OUT>
+int launch_skinny_cfg(const GemmArgs &g, hipStream_t st)
+{
+    constexpr int lds = NWAVE * STAGES * (8192 + XJ * 2048);
+    static_assert(lds >= NWAVE * 4096, "room for the partial tiles");
+    static bool done = false;
+    const int blocks = (g.N + 31) / 32;
+    return launch_with_lds(linear_skinny_kernel<NWAVE, STAGES, XJ, F32OUT>, done, lds, blocks, 64 * NWAVE, g, st,
+                           "linear_skinny_kernel");
+}
+
+template <bool F32OUT>
+int launch_skinny(const GemmArgs &g, hipStream_t st)
+{
+    // Two waves and two ring slots per workgroup measured best: the small LDS
+    // footprint keeps every workgroup of the grid resident at once, and that
+    // parallelism hides latency better than a deeper ring per wave does.
+    if (g.M <= 8)
+        return launch_skinny_cfg<2, 2, 1, F32OUT>(g, st);
+    if (g.M <= 16)
+        return launch_skinny_cfg<2, 2, 2, F32OUT>(g, st);
+    return launch_skinny_cfg<2, 2, 4, F32OUT>(g, st);
+}
+
 template <bool F32OUT>
 int launch_gemm(const GemmArgs &g, hipStream_t st)
 {
@@ -646,6 +847,8 @@ int launch_gemm(const GemmArgs &g, hipStream_t st)
         hipLaunchKernelGGL((gemm_i8_naive_kernel<F32OUT>), grid, dim3(256), 0, st, g);
         return check_launch("gemm_i8_naive_kernel");
     }
+    if (g.K % 256 == 0 && g.M <= 32 && g.N >= 2048 && !getenv("VTL_HIP_GEMM_CONFIG"))
+        return launch_skinny<F32OUT>(g, st);  // weight streaming: enough row blocks to fill the chip
     if (g.K % 128 == 0) {
         int idx, splits;
         choose_config(g.M, g.N, g.K, idx, splits);
