@@ -135,3 +135,49 @@ def test_square_gemm_config_full_size(hip):
     assert np.array_equal(y, want)
     for h in (A, B, Cm, B1, B2, C1, C2, dsa, dsb, dbias):
         h.release()
+
+
+# Shapes chosen to reach every kernel family: the weight-streaming kernel
+# (M <= 32, N >= 2048, K % 256 == 0) with ragged N and M, split-K launches
+# (few output tiles, long K) with uneven K ranges, and the register-staged
+# tile kernel (K % 128 != 0).
+ROUTED_SHAPES = [(1, 2048, 256), (3, 2050, 256), (8, 2048, 4096), (9, 2048, 768), (16, 2047, 1280),
+                 (17, 2077, 1280), (32, 4096, 512), (31, 14336, 256), (5, 3001, 4096),
+                 (256, 1024, 4096), (256, 512, 11008), (64, 128, 11008), (128, 256, 8192), (40, 200, 5504),
+                 (100, 300, 1360), (256, 256, 1040)]
+
+
+@pytest.mark.parametrize("mnk", ROUTED_SHAPES)
+def test_every_kernel_family_matches_oracle(hip, mnk):
+    m, n, k = mnk
+    a, bt, sa, sb, bias = workloads.square_int8_gemm(m, n, k, seed=m * 131 + n * 7 + k)
+    ref = oracle.gemm_i8_i32(a, bt, threads=CPU_THREADS)
+    assert np.array_equal(_gemm(a, bt), ref)
+    A, B, dsa, dsb, dbias = dev(a), dev(bt), dev(sa), dev(sb), dev(bias)
+    for relu, b_dev, b_host in ((True, dbias, bias), (False, None, None)):
+        y = linear_i8_hip(A, dsa, B, dsb, b_dev, relu=relu)
+        got = y.cpu()
+        want = oracle.epilogue(ref, sa, sb, b_host, relu=relu)
+        assert rel_err(got, want) <= F32_REL_TOL and np.array_equal(got, want)
+        y.release()
+    for h in (A, B, dsa, dsb, dbias):
+        h.release()
+
+
+def test_forced_split_k_is_exact(hip, monkeypatch):
+    """Every tile configuration with 1, 2, 3 and 8 K ranges gives the same int32 result."""
+    m, n, k = 96, 384, 2432          # 19 K steps of 128: uneven ranges for every split count
+    a, bt, sa, sb, bias = workloads.square_int8_gemm(m, n, k, seed=77)
+    ref = oracle.gemm_i8_i32(a, bt, threads=CPU_THREADS)
+    want = oracle.epilogue(ref, sa, sb, bias)
+    A, B, dsa, dsb, dbias = dev(a), dev(bt), dev(sa), dev(sb), dev(bias)
+    for idx in range(5):
+        for splits in (1, 2, 3, 8):
+            monkeypatch.setenv("VTL_HIP_GEMM_CONFIG", f"{idx},{splits}")
+            assert np.array_equal(_gemm(a, bt), ref), (idx, splits)
+            y = linear_i8_hip(A, dsa, B, dsb, dbias)
+            assert np.array_equal(y.cpu(), want), (idx, splits)
+            y.release()
+    monkeypatch.delenv("VTL_HIP_GEMM_CONFIG")
+    for h in (A, B, dsa, dsb, dbias):
+        h.release()

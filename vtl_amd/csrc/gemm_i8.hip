@@ -680,28 +680,35 @@ int launch_with_lds(Kern kern, bool &attr_done, int lds, int tiles, int threads,
     return check_launch(name);
 }
 
-// Scratch for split-K partial sums, owned by the library, grown on demand and
-// kept until the process ends (one host thread per device).
+// Scratch for split-K partial sums, owned by the library: one buffer per
+// device, grown on demand and kept until the process ends (one host thread per
+// device).
 int32_t *splitk_workspace(size_t bytes)
 {
-    static int32_t *buf = nullptr;
-    static size_t cap = 0;
-    if (bytes > cap) {
-        if (buf) {
+    constexpr int kMaxDevices = 64;
+    static int32_t *buf[kMaxDevices] = {};
+    static size_t cap[kMaxDevices] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    if (bytes > cap[dev]) {
+        if (buf[dev]) {
             (void)hipStreamSynchronize(current_stream());
-            (void)hipFree(buf);
-            buf = nullptr;
-            cap = 0;
+            (void)hipFree(buf[dev]);
+            buf[dev] = nullptr;
+            cap[dev] = 0;
         }
         const size_t want = bytes < (size_t(32) << 20) ? (size_t(32) << 20) : bytes;
-        if (hipMalloc(reinterpret_cast<void **>(&buf), want) != hipSuccess) {
+        if (hipMalloc(reinterpret_cast<void **>(&buf[dev]), want) != hipSuccess) {
             (void)hipGetLastError();
-            buf = nullptr;
+            buf[dev] = nullptr;
             return nullptr;
         }
-        cap = want;
+        cap[dev] = want;
     }
-    return buf;
+    return buf[dev];
 }
 
 template <int BM, int BN, int BK, int NSTAGE, int WR, int WC, bool F32OUT>
