@@ -34,7 +34,7 @@ PEAK_HBM_GBPS = 8000.0       # HBM3E, MI355X published
 # HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # script, each counter scaled by its reading for the 1 GiB copy_kernel (x2.000 and
 # x0.999); figures and commands in profiles/bench_pmc_traffic.md.
-PMC_TRAFFIC_BYTES = {"linear": 178.6e6, "quantize": 1342.6e6, "dequantize": 1342.7e6}
+PMC_TRAFFIC_BYTES = {"linear": 168.1e6, "quantize": 1342.6e6, "dequantize": 1342.7e6}
 
 
 class Timer:
