@@ -33,7 +33,7 @@ PEAK_HBM_GBPS = 8000.0       # HBM3E, MI355X published
 
 # HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # script, each counter scaled by its reading for the 1 GiB copy_kernel (x2.000 and
-# x0.999); figures and commands in profiles/bench_pmc_traffic.md.
+# x0.999); the summary of those runs is kept with the other profiler summaries.
 PMC_TRAFFIC_BYTES = {"linear": 168.1e6, "quantize": 1342.6e6, "dequantize": 1342.7e6}
 
 
@@ -279,7 +279,7 @@ def main() -> int:
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 "
-              "(the multi-GPU sharding is described in DESIGN.md, not built)", file=sys.stderr)
+              "(sharding across GPUs is a design note only; nothing multi-GPU is built)", file=sys.stderr)
         return 2
     if capi.device_count() < 1:
         print("bench.py: no HIP device visible", file=sys.stderr)

@@ -128,7 +128,15 @@ __global__ __launch_bounds__(T) void absmax_rows_kernel(const float *__restrict_
     if constexpr (VEC == 4) {
         const float4_t *xv = reinterpret_cast<const float4_t *>(xr);
         const int64_t nv = cols >> 2;
-        for (int64_t i = threadIdx.x; i < nv; i += T)
+        int64_t i = threadIdx.x;
+        for (; i + 3 * T < nv; i += 4 * T) {  // four independent loads in flight per lane
+            const float4_t v0 = __builtin_nontemporal_load(xv + i);
+            const float4_t v1 = __builtin_nontemporal_load(xv + i + T);
+            const float4_t v2 = __builtin_nontemporal_load(xv + i + 2 * T);
+            const float4_t v3 = __builtin_nontemporal_load(xv + i + 3 * T);
+            m = absmax4(absmax4(absmax4(absmax4(m, v0), v1), v2), v3);
+        }
+        for (; i < nv; i += T)
             m = absmax4(m, xv[i]);
     } else {
         for (int64_t i = threadIdx.x; i < cols; i += T)
@@ -152,7 +160,15 @@ __global__ __launch_bounds__(T) void absmax_flat_kernel(const float *__restrict_
     if (vec_ok) {
         const float4_t *xv = reinterpret_cast<const float4_t *>(x);
         const int64_t nv = n >> 2;
-        for (int64_t i = tid; i < nv; i += stride)
+        int64_t i = tid;
+        for (; i + 3 * stride < nv; i += 4 * stride) {
+            const float4_t v0 = __builtin_nontemporal_load(xv + i);
+            const float4_t v1 = __builtin_nontemporal_load(xv + i + stride);
+            const float4_t v2 = __builtin_nontemporal_load(xv + i + 2 * stride);
+            const float4_t v3 = __builtin_nontemporal_load(xv + i + 3 * stride);
+            m = absmax4(absmax4(absmax4(absmax4(m, v0), v1), v2), v3);
+        }
+        for (; i < nv; i += stride)
             m = absmax4(m, xv[i]);
         if (tid < (n & 3))
             m = fmaxf(m, fabsf(x[(nv << 2) + tid]));
@@ -480,7 +496,10 @@ int vtl_hip_absmax_f32(const float *x, int64_t rows, int64_t cols, int per_row, 
         if (cols == 0)
             return launch_fill_zero(absmax_out, rows, s);
         const bool vec = (cols % 4 == 0) && aligned(x, 16);
-        if (vec && cols >= 4096)
+        if (vec && cols >= 8192)
+            hipLaunchKernelGGL((absmax_rows_kernel<512, 4>), dim3((unsigned)rows), dim3(512), 0, s, x,
+                               cols, absmax_out);
+        else if (vec && cols >= 1024)
             hipLaunchKernelGGL((absmax_rows_kernel<256, 4>), dim3((unsigned)rows), dim3(256), 0, s, x,
                                cols, absmax_out);
         else if (vec)
