@@ -10,6 +10,8 @@
 #include <stdio.h>
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "common.hpp"
 
 using namespace vtlhip;
@@ -97,17 +99,18 @@ __device__ __forceinline__ void epilogue(v16i (&acc)[WM / 32][WN / 32], const Ge
     const int col_in = lane & 31, row_in = (lane >> 5) * 4;
     const int M = g.M, N = g.N;
     if constexpr (!F32OUT) {
+        int32_t *tile_out = reinterpret_cast<int32_t *>(g.out) + ((int64_t)m0 * N + n0);
 #pragma unroll
         for (int j = 0; j < TN; j++) {
-            const int n = n0 + wc * WN + j * 32 + col_in;
+            const int nl = wc * WN + j * 32 + col_in;
 #pragma unroll
             for (int i = 0; i < TM; i++) {
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
-                    const int m = m0 + wr * WM + i * 32 + 8 * (r >> 2) + row_in + (r & 3);
-                    if (EDGE && (m >= M || n >= N))
+                    const int ml = wr * WM + i * 32 + 8 * (r >> 2) + row_in + (r & 3);
+                    if (EDGE && (m0 + ml >= M || n0 + nl >= N))
                         continue;
-                    reinterpret_cast<int32_t *>(g.out)[(int64_t)m * N + n] = acc[i][j][r];
+                    tile_out[(unsigned)ml * (unsigned)N + (unsigned)nl] = acc[i][j][r];
                 }
             }
         }
@@ -126,38 +129,54 @@ __device__ __forceinline__ void epilogue(v16i (&acc)[WM / 32][WN / 32], const Ge
             s_bias[t] = g.bias ? g.bias[n] : 0.0f;
         }
         __syncthreads();
-        const bool has_bias = g.bias != nullptr;
-        const bool relu = g.relu != 0;
+        // The bias / ReLU switches are uniform: branch once, not per element.
+        auto store_tile = [&](auto has_bias_t, auto relu_t) {
+            constexpr bool HAS_BIAS = decltype(has_bias_t)::value;
+            constexpr bool RELU = decltype(relu_t)::value;
+            // uniform tile origin + 32-bit in-tile offsets keep the address math to one add per store
+            float *tile_out = reinterpret_cast<float *>(g.out) + ((int64_t)m0 * N + n0);
 #pragma unroll
-        for (int j = 0; j < TN; j++) {
-            const int nl = wc * WN + j * 32 + col_in;
-            const int n = n0 + nl;
-            const float w = s_sw[nl];
-            const float bv = s_bias[nl];
+            for (int j = 0; j < TN; j++) {
+                const int nl = wc * WN + j * 32 + col_in;
+                const float w = s_sw[nl];
+                const float bv = s_bias[nl];
 #pragma unroll
-            for (int i = 0; i < TM; i++) {
+                for (int i = 0; i < TM; i++) {
 #pragma unroll
-                for (int rq = 0; rq < 4; rq++) {
-                    const int ml = wr * WM + i * 32 + 8 * rq + row_in;
-                    const f4 a4 = *reinterpret_cast<const f4 *>(s_sa + ml);
+                    for (int rq = 0; rq < 4; rq++) {
+                        const int ml = wr * WM + i * 32 + 8 * rq + row_in;
+                        const f4 a4 = *reinterpret_cast<const f4 *>(s_sa + ml);
 #pragma unroll
-                    for (int k = 0; k < 4; k++) {
-                        const int m = m0 + ml + k;
-                        if (EDGE && (m >= M || n >= N))
-                            continue;
-                        const float s = a4[k] * w;
-                        float y = (float)acc[i][j][rq * 4 + k] * s;
-                        if (has_bias)
-                            y = y + bv;
-                        if (relu && y < 0.0f)
-                            y = 0.0f;
-                        reinterpret_cast<float *>(g.out)[(int64_t)m * N + n] = y;
+                        for (int k = 0; k < 4; k++) {
+                            if (EDGE && (m0 + ml + k >= M || n0 + nl >= N))
+                                continue;
+                            const float s = a4[k] * w;
+                            float y = (float)acc[i][j][rq * 4 + k] * s;
+                            if (HAS_BIAS)
+                                y = y + bv;
+                            if (RELU && y < 0.0f)
+                                y = 0.0f;
+                            tile_out[(unsigned)(ml + k) * (unsigned)N + (unsigned)nl] = y;
+                        }
+                        // keep the compiler from hoisting every scale read of the tile to the
+                        // top of the epilogue, which costs more registers than there are
+                        asm volatile("" ::: "memory");
                     }
-                    // keep the compiler from hoisting every scale read of the tile to the
-                    // top of the epilogue, which costs more registers than there are
-                    asm volatile("" ::: "memory");
                 }
             }
+        };
+        using T_ = std::true_type;
+        using F_ = std::false_type;
+        if (g.bias != nullptr) {
+            if (g.relu)
+                store_tile(T_{}, T_{});
+            else
+                store_tile(T_{}, F_{});
+        } else {
+            if (g.relu)
+                store_tile(F_{}, T_{});
+            else
+                store_tile(F_{}, F_{});
         }
     }
 }
