@@ -133,3 +133,29 @@ def test_session_reuses_buffers_on_second_forward(hip):
     assert s.ensure("dynquant", 1) is buf and np.array_equal(y1, y2)
     s.release()
     layer.release()
+
+
+@pytest.mark.parametrize("nk", [(2048, 256), (2050, 512), (3001, 4096), (2077, 1280)])
+def test_single_token_fused_decode_equals_two_launch_path(hip, nk, monkeypatch):
+    """M = 1 takes the kernel that quantizes the token itself; it must give the
+    bits of the quantize-then-linear path and of the oracle."""
+    n, k = nk
+    rng = np.random.Generator(np.random.Philox(n + k))
+    x = rng.standard_normal((1, k), dtype=np.float32)
+    x[0, :4] = [0.5, 1.5, -2.5, 3.5]
+    w = rng.integers(-127, 128, (n, k), dtype=np.int8)
+    sw = (rng.uniform(0.5, 1.5, n) * 1e-3).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    X, W, SW, B = dev(x), dev(w), dev(sw), dev(bias)
+    want = oracle.linear_f32_dynquant(x, w, sw, bias, relu=True, threads=CPU_THREADS)
+    fused = linear_f32_dynquant_hip(X, W, SW, B, relu=True).cpu()
+    monkeypatch.setenv("VTL_HIP_NO_FUSED_DECODE", "1")
+    plain = linear_f32_dynquant_hip(X, W, SW, B, relu=True).cpu()
+    assert np.array_equal(fused, want) and np.array_equal(plain, want)
+    # degenerate token: all zeros -> scale 0 -> output is the bias (ReLU applied)
+    Z = dev(np.zeros((1, k), np.float32))
+    monkeypatch.delenv("VTL_HIP_NO_FUSED_DECODE")
+    got = linear_f32_dynquant_hip(Z, W, SW, B, relu=False).cpu()
+    assert np.array_equal(got, oracle.linear_f32_dynquant(np.zeros((1, k), np.float32), w, sw, bias))
+    for h in (X, W, SW, B, Z):
+        h.release()
