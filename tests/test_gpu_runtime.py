@@ -1,0 +1,90 @@
+"""Device, memory, transfer, stream and timing entry points on a real device
+(the calls HipStorage makes where CudaStorage calls cudaMalloc / cudaMemcpy /
+cudaFree, storage/cuda_d_cuda.v:32-102)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from helpers import d2h, h2d, raw_device_buffer
+from vtl_amd import capi
+from vtl_amd.storage import HipParams, HipStorage
+from vtl_amd.tensor import HipTensor
+
+pytestmark = pytest.mark.gpu
+
+
+def test_device_queries(hip):
+    assert capi.device_count() >= 1
+    name, cus, mhz = capi.device_info()
+    assert "gfx950" in name and cus == 256 and mhz > 1000
+    assert capi.status("vtl_hip_set_device", capi.device_count() + 3) == capi.ERR_NO_DEVICE
+    assert capi.status("vtl_hip_set_device", -1) == capi.ERR_NO_DEVICE
+    with pytest.raises(capi.VtlHipError) as ei:
+        HipStorage.empty(4, np.float32, HipParams(device_id=99))
+    assert ei.value.status == capi.ERR_NO_DEVICE
+
+
+def test_storage_round_trip_and_release(hip):
+    rng = np.random.default_rng(0)
+    for dtype in (np.float32, np.int8, np.int32):
+        a = (rng.standard_normal(1000) * 50).astype(dtype)
+        st = HipStorage.from_cpu(a)
+        assert st.count == 1000 and st.size == a.nbytes and st.ptr
+        assert st.hip() is st
+        assert np.array_equal(st.cpu(), a) and np.array_equal(st.to_array(), a)
+        st.release()
+        assert st.ptr == 0
+        st.release()                                  # releasing twice is harmless
+    empty = HipStorage.from_cpu(np.zeros(0, np.float32))
+    assert empty.count == 0 and empty.cpu().size == 0
+    t = HipTensor.from_host(np.arange(12, dtype=np.float32).reshape(3, 4))
+    assert t.shape == [3, 4] and t.strides == [4, 1] and t.hip() is t
+    assert np.array_equal(t.cpu(), np.arange(12, dtype=np.float32).reshape(3, 4))
+    t.release()
+
+
+def test_memset_and_device_to_device_copy(hip):
+    n = 1 << 20
+    a, b = raw_device_buffer(n + 64), raw_device_buffer(n + 64)
+    capi.call("vtl_hip_memset", a.ptr, 0x5A, n)
+    capi.call("vtl_hip_memcpy_d2d", b.ptr, a.ptr, n)          # 16-byte aligned: the library's copy kernel
+    assert np.all(d2h(b.ptr, n, np.uint8) == 0x5A)
+    src = np.arange(1001, dtype=np.uint8)
+    h2d(a.ptr + 3, src)
+    capi.call("vtl_hip_memcpy_d2d", b.ptr + 5, a.ptr + 3, src.size)   # unaligned, odd size: runtime copy
+    capi.call("vtl_hip_sync")
+    assert np.array_equal(d2h(b.ptr + 5, src.size, np.uint8), src)
+    a.release()
+    b.release()
+
+
+def test_events_time_a_kernel(hip):
+    e0, e1 = C.c_void_p(), C.c_void_p()
+    capi.call("vtl_hip_event_create", C.byref(e0))
+    capi.call("vtl_hip_event_create", C.byref(e1))
+    x = HipTensor.from_host(np.ones((2048, 4096), np.float32))
+    capi.call("vtl_hip_event_record", e0)
+    q, s = x.quantize_i8(0)
+    capi.call("vtl_hip_event_record", e1)
+    ms = C.c_float(-1.0)
+    capi.call("vtl_hip_event_elapsed_ms", e0, e1, C.byref(ms))
+    assert 0.0 < ms.value < 100.0
+    assert np.all(q.cpu() == 127) and np.all(s.cpu() == np.float32(1.0) / np.float32(127.0))
+    capi.call("vtl_hip_event_destroy", e0)
+    capi.call("vtl_hip_event_destroy", e1)
+    for h in (x, q, s):
+        h.release()
+
+
+def test_unsupported_shapes_return_status(hip):
+    buf = raw_device_buffer(4096)
+    assert capi.status("vtl_hip_gemm_i8_i32", buf.ptr, buf.ptr, buf.ptr, 4, 4, 0) == capi.ERR_UNSUPPORTED
+    assert capi.status("vtl_hip_linear_i8_f32", buf.ptr, buf.ptr, 1, buf.ptr, buf.ptr, 1, None, buf.ptr,
+                       4, 4, 0, 0) == capi.ERR_UNSUPPORTED
+    # workspace too small / misaligned for the dynamic-quantization entry point
+    assert capi.status("vtl_hip_linear_f32_dynquant", buf.ptr, buf.ptr, buf.ptr, None, buf.ptr, 8, 8, 64, 0,
+                       buf.ptr, 16) == capi.ERR_INVALID_ARG
+    assert capi.status("vtl_hip_linear_f32_dynquant", buf.ptr, buf.ptr, buf.ptr, None, buf.ptr, 8, 8, 64, 0,
+                       buf.ptr + 4, 4000) == capi.ERR_INVALID_ARG
+    buf.release()
