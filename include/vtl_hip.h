@@ -133,6 +133,45 @@ int vtl_hip_linear_f32_dynquant(const float *X, const int8_t *Wq, const float *s
                                 const float *bias, float *Y, int M, int N, int K, int relu,
                                 void *workspace, size_t workspace_bytes);
 
+/* ---- f32 / f64 matmul with f64 accumulation ------------------------------ */
+
+/* C[M,N] = op(A) . op(B) with every product and sum in f64 and one rounding
+ * to the tensor's type: la.matmul (la/la.v:38-55: as_f64 -> f64 GEMM ->
+ * as_f32) and gate_matmul (autograd/gates_blas.v:6-23).  trans_a == 0: A is
+ * [M,K] row-major; otherwise A is stored [K,M] and used as its transpose (the
+ * caller's `.t()`, gates_blas.v:43-48).  trans_b == 0: B is [K,N] row-major;
+ * otherwise B is stored [N,K].  All matrices dense row-major.  K == 0 gives
+ * zeros. */
+int vtl_hip_matmul_f32(const float *A, const float *B, float *C, int M, int N, int K,
+                       int trans_a, int trans_b);
+int vtl_hip_matmul_f64(const double *A, const double *B, double *C, int M, int N, int K,
+                       int trans_a, int trans_b);
+
+/* The unquantized Linear forward, y = matmul(x, W^T) + b with W as stored
+ * [N,K] (linear_forward_f32_cpu nn/layers/linear_forward_f32.v:16-18, f64
+ * twin linear_forward_f64.v:7-26): matmul as above, then the bias added in the
+ * tensor's type (Tensor.add, math_op.v:9-21); bias may be NULL; ReLU if
+ * relu != 0. */
+int vtl_hip_linear_f32(const float *X, const float *W, const float *bias, float *Y,
+                       int M, int N, int K, int relu);
+int vtl_hip_linear_f64(const double *X, const double *W, const double *bias, double *Y,
+                       int M, int N, int K, int relu);
+
+/* out[c] = sum_r x[r,c] in f64, rounded once: la.matmul(ones[1,rows], x), the
+ * bias gradient of nn/gates/layers/linear.v:75-79. */
+int vtl_hip_colsum_f32(const float *x, int64_t rows, int64_t cols, float *out);
+int vtl_hip_colsum_f64(const double *x, int64_t rows, int64_t cols, double *out);
+
+/* LinearGate.backward (nn/gates/layers/linear.v:57-79; the reference's device
+ * forms: linear_backward_f64 autograd_cuda/linear_backward_cuda_d_cuda.v:9-36,
+ * linear_backward_vulkan_f32 via linear_gate_backward_f32_d_vulkan.v:8-13):
+ * dx[M,K] = grad[M,N] . W[N,K], dw[N,K] = grad^T . x[M,K], db[N] = column sums
+ * of grad.  Any of dx, dw, db may be NULL (gradient not required). */
+int vtl_hip_linear_backward_f32(const float *grad, const float *x, const float *W, float *dx,
+                                float *dw, float *db, int M, int N, int K);
+int vtl_hip_linear_backward_f64(const double *grad, const double *x, const double *W, double *dx,
+                                double *dw, double *db, int M, int N, int K);
+
 /* ReLU in place on the device (nn/internal/activation.v:63-70,
  * relu_cuda tensor_cuda_d_cuda.v:205-235). */
 int vtl_hip_relu_f32(float *x, int64_t n);

@@ -47,6 +47,12 @@ def lib() -> C.CDLL:
         "vtl_ref_linear_f32_dynquant": (None, [vp, vp, vp, vp, vp, i64, i64, i64, ci, ci]),
         "vtl_ref_relu_f32": (None, [vp, i64]),
         "vtl_ref_linear_f32_via_f64": (None, [vp, vp, vp, vp, i64, i64, i64]),
+        "vtl_ref_matmul_f32": (None, [vp, vp, vp, i64, i64, i64, ci, ci, ci]),
+        "vtl_ref_matmul_f64": (None, [vp, vp, vp, i64, i64, i64, ci, ci, ci]),
+        "vtl_ref_colsum_f32": (None, [vp, i64, i64, vp]),
+        "vtl_ref_colsum_f64": (None, [vp, i64, i64, vp]),
+        "vtl_ref_linear_backward_f32": (None, [vp, vp, vp, vp, vp, vp, i64, i64, i64, ci]),
+        "vtl_ref_linear_backward_f64": (None, [vp, vp, vp, vp, vp, vp, i64, i64, i64, ci]),
         "vtl_ref_quantize_f32_i8_mt": (None, [vp, i64, i64, ci, vp, vp, ci]),
         "vtl_ref_dequantize_i8_f32_mt": (None, [vp, vp, i64, i64, ci, vp, ci]),
         "vtl_ref_max_threads": (ci, []),
@@ -188,3 +194,49 @@ def linear_f32_via_f64(X, W, bias) -> np.ndarray:
     Y = np.empty((M, N), np.float32)
     lib().vtl_ref_linear_f32_via_f64(_p(X), _p(W), _p(b), _p(Y), M, N, K)
     return Y
+
+
+def _suffix(dtype) -> str:
+    dt = np.dtype(dtype)
+    if dt == np.float32:
+        return "f32"
+    if dt == np.float64:
+        return "f64"
+    raise TypeError(f"matmul oracle covers float32 and float64, not {dt}")
+
+
+def matmul(a: np.ndarray, b: np.ndarray, trans_a: bool = False, trans_b: bool = False,
+           threads: int = 1) -> np.ndarray:
+    """op(a) . op(b) through f64, rounded once to the operands' dtype."""
+    sfx = _suffix(a.dtype)
+    a = _c(a, a.dtype)
+    b = _c(b, a.dtype)
+    M, K = (a.shape[1], a.shape[0]) if trans_a else a.shape
+    K2, N = (b.shape[1], b.shape[0]) if trans_b else b.shape
+    assert K == K2, (a.shape, b.shape, trans_a, trans_b)
+    c = np.empty((M, N), a.dtype)
+    getattr(lib(), f"vtl_ref_matmul_{sfx}")(_p(a), _p(b), _p(c), M, N, K, int(trans_a), int(trans_b),
+                                            threads)
+    return c
+
+
+def colsum(x: np.ndarray) -> np.ndarray:
+    sfx = _suffix(x.dtype)
+    x = _c(x, x.dtype)
+    out = np.empty(x.shape[1], x.dtype)
+    getattr(lib(), f"vtl_ref_colsum_{sfx}")(_p(x), x.shape[0], x.shape[1], _p(out))
+    return out
+
+
+def linear_backward(grad: np.ndarray, x: np.ndarray, w: np.ndarray, threads: int = 1):
+    """(dx[M,K], dw[N,K], db[N]) of y = x.W^T + b for the upstream gradient grad[M,N]."""
+    sfx = _suffix(grad.dtype)
+    dt = grad.dtype
+    grad, x, w = _c(grad, dt), _c(x, dt), _c(w, dt)
+    M, N = grad.shape
+    K = x.shape[1]
+    assert x.shape == (M, K) and w.shape == (N, K)
+    dx, dw, db = np.empty((M, K), dt), np.empty((N, K), dt), np.empty(N, dt)
+    getattr(lib(), f"vtl_ref_linear_backward_{sfx}")(_p(grad), _p(x), _p(w), _p(dx), _p(dw), _p(db),
+                                                     M, N, K, threads)
+    return dx, dw, db

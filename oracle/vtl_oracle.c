@@ -31,6 +31,17 @@
  *                               Summation order of the un-vendored VSL GEMM
  *                               is unknown: parity unpinned beyond f64
  *                               rounding error.
+ *   vtl_ref_matmul_f32/_f64     la/la_test.v:30-37 (I.B = B), numpy f64
+ *                               matmul on explicit transposes, integer-valued
+ *                               operands (every order of summation exact)
+ *                               against numpy int64 matmul, the literals of
+ *                               benchmarks/vs_numpy/matmul_bench.v:28-33 in
+ *                               closed form.  Same caveat on VSL's order.
+ *   vtl_ref_colsum_f32/_f64     math.fsum (exact sum, one rounding).
+ *   vtl_ref_linear_backward_*   autograd_cuda/device_session_test.v:52-60
+ *                               operands worked by hand (dx = [0.3, 0.45,
+ *                               0.6], dw = [[1,2,3],[0.5,1,1.5]], db = grad),
+ *                               central finite differences of the f64 forward.
  */
 #include "vtl_oracle.h"
 
@@ -221,6 +232,53 @@ void vtl_ref_linear_f32_via_f64(const float *X, const float *W, const float *bia
         }
     }
 }
+
+#define VTL_REF_MATMUL(NAME, T)                                                              \
+    void NAME(const T *A, const T *B, T *C, int64_t M, int64_t N, int64_t K, int trans_a,     \
+              int trans_b, int threads)                                                       \
+    {                                                                                         \
+        const int64_t a_rs = trans_a ? 1 : K, a_ks = trans_a ? M : 1;                         \
+        const int64_t b_ks = trans_b ? 1 : N, b_cs = trans_b ? K : 1;                         \
+        (void)threads;                                                                        \
+        _Pragma("omp parallel for schedule(static) num_threads(threads > 1 ? threads : 1)")   \
+        for (int64_t m = 0; m < M; m++) {                                                     \
+            for (int64_t n = 0; n < N; n++) {                                                 \
+                double acc = 0.0;                                                             \
+                for (int64_t k = 0; k < K; k++)                                               \
+                    acc += (double)A[m * a_rs + k * a_ks] * (double)B[k * b_ks + n * b_cs];   \
+                C[m * N + n] = (T)acc; /* as_f32 for f32, la/la.v:51-53 */                    \
+            }                                                                                 \
+        }                                                                                     \
+    }
+VTL_REF_MATMUL(vtl_ref_matmul_f32, float)
+VTL_REF_MATMUL(vtl_ref_matmul_f64, double)
+
+#define VTL_REF_COLSUM(NAME, T)                                   \
+    void NAME(const T *x, int64_t rows, int64_t cols, T *out)     \
+    {                                                             \
+        for (int64_t c = 0; c < cols; c++) {                      \
+            double acc = 0.0;                                     \
+            for (int64_t r = 0; r < rows; r++)                    \
+                acc += 1.0 * (double)x[r * cols + c];             \
+            out[c] = (T)acc;                                      \
+        }                                                         \
+    }
+VTL_REF_COLSUM(vtl_ref_colsum_f32, float)
+VTL_REF_COLSUM(vtl_ref_colsum_f64, double)
+
+#define VTL_REF_LINEAR_BACKWARD(NAME, T, MATMUL, COLSUM)                                          \
+    void NAME(const T *grad, const T *x, const T *w, T *dx, T *dw, T *db, int64_t M, int64_t N,    \
+              int64_t K, int threads)                                                              \
+    {                                                                                              \
+        if (dx) /* la.matmul(grad, weight), linear.v:69-70 */                                      \
+            MATMUL(grad, w, dx, M, K, N, 0, 0, threads);                                           \
+        if (dw) /* la.matmul(grad.t(), input), linear.v:72-73 */                                   \
+            MATMUL(grad, x, dw, N, K, M, 1, 0, threads);                                           \
+        if (db) /* la.matmul(ones[1,batch], grad), linear.v:75-79 */                               \
+            COLSUM(grad, M, N, db);                                                                \
+    }
+VTL_REF_LINEAR_BACKWARD(vtl_ref_linear_backward_f32, float, vtl_ref_matmul_f32, vtl_ref_colsum_f32)
+VTL_REF_LINEAR_BACKWARD(vtl_ref_linear_backward_f64, double, vtl_ref_matmul_f64, vtl_ref_colsum_f64)
 
 /* Row-parallel forms of the two bandwidth-bound routines, used only to time
  * the CPU baseline on all host cores.  Same arithmetic per element. */

@@ -98,6 +98,34 @@ void vtl_ref_relu_f32(float *x, int64_t n);
 void vtl_ref_linear_f32_via_f64(const float *X, const float *W, const float *bias, float *Y,
                                 int64_t M, int64_t N, int64_t K);
 
+/* C[M,N] = op(A) . op(B) the way la.matmul (la/la.v:38-55) and gate_matmul
+ * (autograd/gates_blas.v:6-23) compute it: every element widened to f64, a
+ * f64 GEMM (here: k ascending, one f64 accumulator per element), one rounding
+ * to the tensor's type (as_f32 for f32; f64 stays).  trans_a == 0: A is
+ * [M,K] row-major, else A is stored [K,M] (the caller's `.t()`, as in
+ * MatMulGate.backward gates_blas.v:43-48 and LinearGate.backward
+ * nn/gates/layers/linear.v:69-74); same for B ([K,N] / [N,K]).  threads > 1:
+ * OpenMP over rows, same arithmetic.  Summation order inside VSL's GEMM is
+ * unknown: parity unpinned beyond f64 rounding error. */
+void vtl_ref_matmul_f32(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K,
+                        int trans_a, int trans_b, int threads);
+void vtl_ref_matmul_f64(const double *A, const double *B, double *C, int64_t M, int64_t N, int64_t K,
+                        int trans_a, int trans_b, int threads);
+
+/* out[c] = sum over rows of x[r,c], summed in f64 and rounded once:
+ * la.matmul(ones[1,M], grad), nn/gates/layers/linear.v:75-79. */
+void vtl_ref_colsum_f32(const float *x, int64_t rows, int64_t cols, float *out);
+void vtl_ref_colsum_f64(const double *x, int64_t rows, int64_t cols, double *out);
+
+/* LinearGate.backward (nn/gates/layers/linear.v:57-79; f64 twin
+ * autograd_cuda/linear_backward_f64.v): dx[M,K] = grad[M,N] . W[N,K],
+ * dw[N,K] = grad^T . x[M,K], db[N] = ones[1,M] . grad.  Any output may be
+ * NULL (that gradient is not required). */
+void vtl_ref_linear_backward_f32(const float *grad, const float *x, const float *w, float *dx,
+                                 float *dw, float *db, int64_t M, int64_t N, int64_t K, int threads);
+void vtl_ref_linear_backward_f64(const double *grad, const double *x, const double *w, double *dx,
+                                 double *dw, double *db, int64_t M, int64_t N, int64_t K, int threads);
+
 /* Row-parallel forms (same arithmetic), for timing the CPU baseline on all cores. */
 void vtl_ref_quantize_f32_i8_mt(const float *x, int64_t rows, int64_t cols, int per_row,
                                 int8_t *q, float *scale_out, int threads);

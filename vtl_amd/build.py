@@ -9,7 +9,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 REPO_ROOT = os.path.dirname(PKG_DIR)
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libvtlhip.so")
-SOURCES = ["runtime.hip", "quant.hip", "gemm_i8.hip"]
+SOURCES = ["runtime.hip", "quant.hip", "gemm_i8.hip", "matmul_f64acc.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

@@ -48,6 +48,14 @@ SIGNATURES = {
     "vtl_hip_linear_i8_f32": (_ci, [_vp, _vp, _ci, _vp, _vp, _ci, _vp, _vp, _ci, _ci, _ci, _ci]),
     "vtl_hip_linear_f32_dynquant_workspace": (_sz, [_ci, _ci]),
     "vtl_hip_linear_f32_dynquant": (_ci, [_vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp, _sz]),
+    "vtl_hip_matmul_f32": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci]),
+    "vtl_hip_matmul_f64": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci]),
+    "vtl_hip_linear_f32": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci]),
+    "vtl_hip_linear_f64": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci]),
+    "vtl_hip_colsum_f32": (_ci, [_vp, _i64, _i64, _vp]),
+    "vtl_hip_colsum_f64": (_ci, [_vp, _i64, _i64, _vp]),
+    "vtl_hip_linear_backward_f32": (_ci, [_vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci]),
+    "vtl_hip_linear_backward_f64": (_ci, [_vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci]),
     "vtl_hip_relu_f32": (_ci, [_vp, _i64]),
     "vtl_hip_strerror": (C.c_char_p, [_ci]),
     "vtl_hip_last_error": (C.c_char_p, []),

@@ -21,6 +21,12 @@ int check_launch(const char *kernel_name);
 // Streaming copy kernel (quant.hip); false when alignment or size do not qualify.
 bool launch_copy(void *dst, const void *src, size_t bytes, hipStream_t st);
 
+// Device scratch owned by the library (split-K partial sums, partial column
+// sums): one buffer per device, grown on demand and kept until the process
+// ends.  Kernels enqueued on the current stream may use it until the next
+// call that asks for it; nullptr when the allocation fails.
+void *library_workspace(size_t bytes);
+
 constexpr int kWave = 64;
 
 }  // namespace vtlhip

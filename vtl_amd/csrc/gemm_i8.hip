@@ -888,37 +888,6 @@ int launch_with_lds(Kern kern, bool &attr_done, int lds, int tiles, int threads,
     return check_launch(name);
 }
 
-// Scratch for split-K partial sums, owned by the library: one buffer per
-// device, grown on demand and kept until the process ends (one host thread per
-// device).
-int32_t *splitk_workspace(size_t bytes)
-{
-    constexpr int kMaxDevices = 64;
-    static int32_t *buf[kMaxDevices] = {};
-    static size_t cap[kMaxDevices] = {};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
-        (void)hipGetLastError();
-        return nullptr;
-    }
-    if (bytes > cap[dev]) {
-        if (buf[dev]) {
-            (void)hipStreamSynchronize(current_stream());
-            (void)hipFree(buf[dev]);
-            buf[dev] = nullptr;
-            cap[dev] = 0;
-        }
-        const size_t want = bytes < (size_t(32) << 20) ? (size_t(32) << 20) : bytes;
-        if (hipMalloc(reinterpret_cast<void **>(&buf[dev]), want) != hipSuccess) {
-            (void)hipGetLastError();
-            buf[dev] = nullptr;
-            return nullptr;
-        }
-        cap[dev] = want;
-    }
-    return buf[dev];
-}
-
 template <int BM, int BN, int BK, int NSTAGE, int WR, int WC, bool F32OUT>
 int launch_dma(GemmArgs g, int splits, hipStream_t st)
 {
@@ -933,7 +902,8 @@ int launch_dma(GemmArgs g, int splits, hipStream_t st)
         splits = 1;
     g.splits = splits;
     if (splits > 1) {
-        g.partials = splitk_workspace((size_t)splits * (size_t)g.M * (size_t)g.N * sizeof(int32_t));
+        g.partials = static_cast<int32_t *>(
+            vtlhip::library_workspace((size_t)splits * (size_t)g.M * (size_t)g.N * sizeof(int32_t)));
         if (!g.partials)
             return VTL_HIP_ERR_OUT_OF_MEMORY;
     }

@@ -32,6 +32,34 @@ int check_launch(const char *kernel_name)
     return VTL_HIP_OK;
 }
 
+void *library_workspace(size_t bytes)
+{
+    constexpr int kMaxDevices = 64;
+    static void *buf[kMaxDevices] = {};
+    static size_t cap[kMaxDevices] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    if (bytes > cap[dev]) {
+        if (buf[dev]) {
+            (void)hipStreamSynchronize(current_stream());
+            (void)hipFree(buf[dev]);
+            buf[dev] = nullptr;
+            cap[dev] = 0;
+        }
+        const size_t want = bytes < (size_t(32) << 20) ? (size_t(32) << 20) : bytes;
+        if (hipMalloc(&buf[dev], want) != hipSuccess) {
+            (void)hipGetLastError();
+            buf[dev] = nullptr;
+            return nullptr;
+        }
+        cap[dev] = want;
+    }
+    return buf[dev];
+}
+
 }  // namespace vtlhip
 
 using namespace vtlhip;

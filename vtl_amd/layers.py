@@ -23,7 +23,8 @@ import numpy as np
 
 from . import capi
 from .storage import HipParams, HipStorage
-from .tensor import HipTensor, linear_f32_dynquant_hip, linear_i8_hip
+from .tensor import (HipTensor, linear_backward_hip, linear_f32_dynquant_hip, linear_hip, linear_i8_hip,
+                     matmul_hip)
 
 
 # -- nn/layers/hip_config.v (cf. vulkan_config.v:12-24, cuda_config.v:11-23) ----
@@ -47,6 +48,18 @@ def linear_forward_f32_use_hip() -> bool:
 
 PER_TENSOR = "per_tensor"      # one scale for x, one for W
 PER_CHANNEL = "per_channel"    # one scale per row of x (token) and per row of W (output channel)
+
+
+def hip_backward_enabled() -> bool:
+    """Linear gate gradients on the device: VTL_USE_HIP=1 and VTL_HIP_BACKWARD=1
+    (cf. cuda_backward_enabled, autograd_cuda/gpu_config.v:20-23)."""
+    return os.environ.get("VTL_USE_HIP") == "1" and os.environ.get("VTL_HIP_BACKWARD") == "1"
+
+
+def linear_gate_use_hip_backward() -> bool:
+    """Hook asked by LinearGate.backward (cf. linear_gate_use_vulkan_backward,
+    nn/gates/layers/linear_gate_vulkan_hooks_d_vulkan.v:6-8)."""
+    return hip_backward_enabled() and capi.device_count() > 0
 
 
 class HipSession:
@@ -218,3 +231,81 @@ def kaiming_normal(shape, rng: np.random.Generator) -> np.ndarray:
     f0 = shape[0] * int(np.prod(shape[1:]))
     std = np.sqrt(2.0 / f0)
     return (rng.standard_normal(shape) * std).astype(np.float32)
+
+
+# -- la.matmul / Linear forward and backward in full precision -----------------
+
+def _as_float_matrix(t, what: str) -> np.ndarray:
+    a = np.asarray(t)
+    if a.dtype not in (np.float32, np.float64):
+        raise TypeError(f"{what}: f32 or f64 tensor expected, got {a.dtype}")
+    if a.ndim != 2:
+        raise ValueError("Matrix expected")
+    return a
+
+
+def matmul_hip_host(a: np.ndarray, b: np.ndarray) -> np.ndarray:
+    """`la.matmul[T](a, b)` (la/la.v:38-55) through the device: upload both
+    operands, f64-accumulating matmul, download.  Shape errors carry the
+    reference's message."""
+    a = _as_float_matrix(a, "matmul")
+    b = _as_float_matrix(b, "matmul")
+    if a.shape[1] != b.shape[0]:
+        raise ValueError(f"Invalid shapes for matrix multiplication {list(a.shape)} and {list(b.shape)}")
+    a_dev = HipTensor.from_host(a)
+    b_dev = HipTensor.from_host(b.astype(a.dtype, copy=False))
+    try:
+        c_dev = matmul_hip(a_dev, b_dev)
+        try:
+            return c_dev.cpu()
+        finally:
+            c_dev.release()
+    finally:
+        a_dev.release()
+        b_dev.release()
+
+
+def linear_forward_hip_exact(x: np.ndarray, weights: np.ndarray, bias: np.ndarray | None) -> np.ndarray:
+    """The unquantized Linear forward on the device with the arithmetic of
+    linear_forward_f32_cpu (nn/layers/linear_forward_f32.v:16-18): matmul(x, W^T)
+    through f64, then the bias added in the tensor's type."""
+    x = _as_float_matrix(x, "linear")
+    w = _as_float_matrix(weights, "linear").astype(x.dtype, copy=False)
+    x_dev, w_dev = HipTensor.from_host(x), HipTensor.from_host(w)
+    b_dev = None if bias is None else HipTensor.from_host(np.asarray(bias, x.dtype).reshape(1, -1))
+    try:
+        y_dev = linear_hip(x_dev, w_dev, b_dev)
+        try:
+            return y_dev.cpu()
+        finally:
+            y_dev.release()
+    finally:
+        for t in (x_dev, w_dev, b_dev):
+            if t is not None:
+                t.release()
+
+
+def linear_backward_hip_f32(grad: np.ndarray, input: np.ndarray, weight: np.ndarray,
+                            bias_needs_grad: bool):
+    """`linear_backward_hip_f32(grad, input, weight, bias_needs_grad) ![]&vtl.Tensor[f32]`:
+    [d_input, d_weight, d_bias] of a Linear layer, the HIP counterpart of
+    linear_backward_vulkan_f32 (nn/internal/linear_vulkan_backward_d_vulkan.v:9-38)
+    and linear_backward_f64 (autograd_cuda/linear_backward_cuda_d_cuda.v:9-36).
+    d_bias is [1, out_features]: the column sums of grad, or zeros when the bias
+    needs no gradient.  Works for f32 and f64 host tensors alike."""
+    if not hip_backward_enabled():
+        raise RuntimeError("linear_backward_hip_f32: set VTL_USE_HIP=1 and VTL_HIP_BACKWARD=1")
+    g = _as_float_matrix(grad, "linear backward")
+    x = _as_float_matrix(input, "linear backward").astype(g.dtype, copy=False)
+    w = _as_float_matrix(weight, "linear backward").astype(g.dtype, copy=False)
+    g_dev, x_dev, w_dev = HipTensor.from_host(g), HipTensor.from_host(x), HipTensor.from_host(w)
+    outs = []
+    try:
+        outs = linear_backward_hip(g_dev, x_dev, w_dev, need_db=bias_needs_grad)
+        d_in, d_w = outs[0].cpu(), outs[1].cpu()
+        d_b = outs[2].cpu() if bias_needs_grad else np.zeros((1, w.shape[0]), g.dtype)
+        return [d_in, d_w, d_b]
+    finally:
+        for t in (g_dev, x_dev, w_dev, *outs):
+            if t is not None:
+                t.release()

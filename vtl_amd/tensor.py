@@ -212,3 +212,77 @@ def linear_f32_dynquant_hip(x: HipTensor, w_q: HipTensor, sw: HipTensor, bias: H
         if own:
             ws.release()
     return y
+
+
+def _float_suffix(t: HipTensor, what: str) -> str:
+    if t.dtype == np.float32:
+        return "f32"
+    if t.dtype == np.float64:
+        return "f64"
+    raise TypeError(f"{what}: f32 or f64 tensor expected, got {t.dtype}")
+
+
+def matmul_hip(a: HipTensor, b: HipTensor, trans_a: bool = False, trans_b: bool = False) -> HipTensor:
+    """`matmul_hip(a, b) !&HipTensor[T]`: la.matmul (la/la.v:38-55) on the device, f64
+    products and sums, one rounding to T.  trans_a / trans_b take the stored matrix
+    as its transpose, which is how the gates pass `.t()` (autograd/gates_blas.v:43-48)."""
+    sfx = _float_suffix(a, "matmul_hip")
+    if b.dtype != a.dtype:
+        raise TypeError("matmul_hip: operands of one type expected")
+    if not a.is_matrix() or not b.is_matrix():
+        raise ValueError("Matrix expected")
+    m, k = (a.shape[1], a.shape[0]) if trans_a else a.shape
+    k2, n = (b.shape[1], b.shape[0]) if trans_b else b.shape
+    if k != k2:
+        raise ValueError(f"Invalid shapes for matrix multiplication {[m, k]} and {[k2, n]}")
+    c = HipTensor.empty([m, n], a.dtype, HipParams(a.data.device_id))
+    capi.call(f"vtl_hip_matmul_{sfx}", a.ptr, b.ptr, c.ptr, m, n, k, int(trans_a), int(trans_b))
+    return c
+
+
+def linear_hip(x: HipTensor, w: HipTensor, bias: HipTensor | None, relu: bool = False) -> HipTensor:
+    """The unquantized Linear forward y = matmul(x, W^T) + b with W as stored [N,K]
+    (linear_forward_f32_cpu, nn/layers/linear_forward_f32.v:16-18)."""
+    sfx = _float_suffix(x, "linear_hip")
+    if w.dtype != x.dtype or (bias is not None and bias.dtype != x.dtype):
+        raise TypeError("linear_hip: operands of one type expected")
+    m, n, k = _matmul_shapes(x, w)
+    if bias is not None and bias.size != n:
+        raise ValueError(f"linear_hip: bias has {bias.size} entries, expected {n}")
+    y = HipTensor.empty([m, n], x.dtype, HipParams(x.data.device_id))
+    capi.call(f"vtl_hip_linear_{sfx}", x.ptr, w.ptr, bias.ptr if bias is not None else None, y.ptr,
+              m, n, k, int(relu))
+    return y
+
+
+def colsum_hip(x: HipTensor) -> HipTensor:
+    """la.matmul(ones[1,rows], x) as [1, cols] (nn/gates/layers/linear.v:75-79)."""
+    sfx = _float_suffix(x, "colsum_hip")
+    if not x.is_matrix():
+        raise ValueError("Matrix expected")
+    out = HipTensor.empty([1, x.shape[1]], x.dtype, HipParams(x.data.device_id))
+    capi.call(f"vtl_hip_colsum_{sfx}", x.ptr, x.shape[0], x.shape[1], out.ptr)
+    return out
+
+
+def linear_backward_hip(grad: HipTensor, x: HipTensor, w: HipTensor, need_dx: bool = True,
+                        need_dw: bool = True, need_db: bool = True):
+    """LinearGate.backward on the device (nn/gates/layers/linear.v:57-79): returns
+    [dx[M,K], dw[N,K], db[1,N]] with None where a gradient is not required."""
+    sfx = _float_suffix(grad, "linear_backward_hip")
+    if x.dtype != grad.dtype or w.dtype != grad.dtype:
+        raise TypeError("linear_backward_hip: operands of one type expected")
+    if not (grad.is_matrix() and x.is_matrix() and w.is_matrix()):
+        raise ValueError("Matrix expected")
+    m, n = grad.shape
+    k = x.shape[1]
+    if x.shape != [m, k] or w.shape != [n, k]:
+        raise ValueError(f"linear_backward_hip: grad {grad.shape}, input {x.shape}, weight {w.shape}")
+    params = HipParams(grad.data.device_id)
+    dx = HipTensor.empty([m, k], grad.dtype, params) if need_dx else None
+    dw = HipTensor.empty([n, k], grad.dtype, params) if need_dw else None
+    db = HipTensor.empty([1, n], grad.dtype, params) if need_db else None
+    capi.call(f"vtl_hip_linear_backward_{sfx}", grad.ptr, x.ptr, w.ptr,
+              dx.ptr if dx is not None else None, dw.ptr if dw is not None else None,
+              db.ptr if db is not None else None, m, n, k)
+    return [dx, dw, db]
