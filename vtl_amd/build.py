@@ -4,11 +4,13 @@ from __future__ import annotations
 import os
 import subprocess
 import sys
+from concurrent.futures import ThreadPoolExecutor
 
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 REPO_ROOT = os.path.dirname(PKG_DIR)
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libvtlhip.so")
+OBJ_DIR = os.path.join(PKG_DIR, "_build")
 SOURCES = ["runtime.hip", "quant.hip", "gemm_i8.hip", "matmul_f64acc.hip"]
 
 HIPCC_FLAGS = [
@@ -16,7 +18,6 @@ HIPCC_FLAGS = [
     "-O3",
     "-std=c++17",
     "-fPIC",
-    "-shared",
     # the f32 epilogue and the quantizer are specified as separately rounded
     # operations: no fused multiply-add contraction
     "-ffp-contract=off",
@@ -26,6 +27,13 @@ HIPCC_FLAGS = [
     "-Wno-unused-function",
 ]
 
+# Flags of single sources.  The f64 MFMA accumulators of the matmul kernel fit
+# the architectural VGPRs; asking for the VGPR form of MFMA keeps the compiler
+# from shuttling them to and from the accumulation registers every k-step.
+SOURCE_FLAGS = {
+    "matmul_f64acc.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+}
+
 
 def hipcc() -> str:
     for cand in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
@@ -34,11 +42,7 @@ def hipcc() -> str:
     return "hipcc"
 
 
-def build_lib(verbose: bool = False, extra_flags: list[str] | None = None) -> str:
-    """Compile every HIP source into vtl_amd/libvtlhip.so."""
-    cmd = [hipcc(), *HIPCC_FLAGS, *(extra_flags or []),
-           "-I", os.path.join(REPO_ROOT, "include"), "-I", CSRC,
-           *[os.path.join(CSRC, s) for s in SOURCES], "-o", LIB_PATH]
+def _run(cmd: list[str], verbose: bool) -> None:
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -47,7 +51,24 @@ def build_lib(verbose: bool = False, extra_flags: list[str] | None = None) -> st
     if res.returncode != 0:
         raise RuntimeError("hipcc failed:\n" + out)
     if verbose and out.strip():
-        print(out)
+        print(out, flush=True)
+
+
+def build_lib(verbose: bool = False, extra_flags: list[str] | None = None) -> str:
+    """Compile every HIP source (one object each, side by side) and link
+    vtl_amd/libvtlhip.so."""
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    includes = ["-I", os.path.join(REPO_ROOT, "include"), "-I", CSRC]
+    objects = [os.path.join(OBJ_DIR, s.replace(".hip", ".o")) for s in SOURCES]
+
+    def compile_one(i: int) -> None:
+        src = SOURCES[i]
+        _run([hipcc(), *HIPCC_FLAGS, *SOURCE_FLAGS.get(src, []), *(extra_flags or []), *includes,
+              "-c", os.path.join(CSRC, src), "-o", objects[i]], verbose)
+
+    with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as pool:
+        list(pool.map(compile_one, range(len(SOURCES))))
+    _run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *objects, "-o", LIB_PATH], verbose)
     return LIB_PATH
 
 
