@@ -38,13 +38,14 @@ struct alignas(16) Vec4 {
 };
 
 // Four consecutive elements of a row-major matrix starting at (row, col);
-// positions outside rows x cols read as zero.
-template <typename T>
+// positions outside rows x cols read as zero.  GUARD == false: the caller
+// knows that every position is inside and 16-byte aligned.
+template <typename T, bool GUARD>
 __device__ __forceinline__ Vec4<T> load4(const T *__restrict__ base, int ld, int rows, int cols, int row,
                                          int col, bool vec_ok)
 {
     Vec4<T> out;
-    if (row < rows && col + 3 < cols && vec_ok) {
+    if (!GUARD || (row < rows && col + 3 < cols && vec_ok)) {
         out = *reinterpret_cast<const Vec4<T> *>(base + (int64_t)row * ld + col);
     } else {
 #pragma unroll
@@ -70,7 +71,7 @@ __device__ __forceinline__ void read_operands(const T *__restrict__ p, double (&
 // One operand tile of BK x BMN elements (k-major in LDS, row stride LDW).
 // KMAJOR: the matrix is stored with the tile's m/n index contiguous ([K, MN]);
 // otherwise it is stored [MN, K] and is transposed on the way into LDS.
-template <typename T, int BK, int BMN, int LDW, bool KMAJOR>
+template <typename T, int BK, int BMN, int LDW, bool KMAJOR, bool GUARD>
 struct OperandTile {
     static constexpr int kGroups = BK * BMN / 4;           // 4-element groups per tile
     static constexpr int kPerThread = (kGroups + 255) / 256;
@@ -88,10 +89,10 @@ struct OperandTile {
                 break;
             if constexpr (KMAJOR) {
                 const int krow = g / (BMN / 4), c4 = g % (BMN / 4);
-                regs[i] = load4<T>(base, mn_total, k_total, mn_total, k0 + krow, mn0 + 4 * c4, vec_ok);
+                regs[i] = load4<T, GUARD>(base, mn_total, k_total, mn_total, k0 + krow, mn0 + 4 * c4, vec_ok);
             } else {
                 const int mn = g % BMN, kc = g / BMN;
-                regs[i] = load4<T>(base, k_total, mn_total, k_total, mn0 + mn, k0 + 4 * kc, vec_ok);
+                regs[i] = load4<T, GUARD>(base, k_total, mn_total, k_total, mn0 + mn, k0 + 4 * kc, vec_ok);
             }
         }
     }
@@ -117,7 +118,9 @@ struct OperandTile {
     }
 };
 
-template <typename T, int BM, int BN, bool TA, bool TB>
+// GUARD == false: M, N, K are whole tiles and every row is 16-byte aligned, so
+// the loads and stores carry no bounds checks and the k-loop is straight-line code.
+template <typename T, int BM, int BN, bool TA, bool TB, bool GUARD>
 __global__ __launch_bounds__(256) void matmul_f64acc_kernel(const MatmulArgs g)
 {
     constexpr int BK = 64 / (int)sizeof(T);   // 16 for f32, 8 for f64
@@ -139,9 +142,9 @@ __global__ __launch_bounds__(256) void matmul_f64acc_kernel(const MatmulArgs g)
     const int r16 = lane & 15, kq = lane >> 4;
 
     // A as op(A)[M,K]: stored [K,M] when transposed (k-major already)
-    OperandTile<T, BK, BM, LDA, TA> ta;
+    OperandTile<T, BK, BM, LDA, TA, GUARD> ta;
     // B as op(B)[K,N]: stored [K,N] when not transposed (k-major already)
-    OperandTile<T, BK, BN, LDB, !TB> tb;
+    OperandTile<T, BK, BN, LDB, !TB, GUARD> tb;
 
     double4_t acc[TM][TN];
 #pragma unroll
@@ -194,13 +197,13 @@ __global__ __launch_bounds__(256) void matmul_f64acc_kernel(const MatmulArgs g)
     T bv[TN];
 #pragma unroll
     for (int j = 0; j < TN; ++j)
-        bv[j] = (bias && col0 + j < g.N) ? bias[col0 + j] : T(0);
+        bv[j] = (bias && (!GUARD || col0 + j < g.N)) ? bias[col0 + j] : T(0);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const int row = m0 + wm + TM * (4 * e + kq) + i;
-            if (row >= g.M)
+            if (GUARD && row >= g.M)
                 continue;
             T out[TN];
 #pragma unroll
@@ -213,7 +216,7 @@ __global__ __launch_bounds__(256) void matmul_f64acc_kernel(const MatmulArgs g)
                 out[j] = y;
             }
             T *dst = C + (int64_t)row * g.N + col0;
-            if (g.vec_c && col0 + TN - 1 < g.N) {
+            if (!GUARD || (g.vec_c && col0 + TN - 1 < g.N)) {
                 if constexpr (TN == 4) {
                     Vec4<T> v;
 #pragma unroll
@@ -315,22 +318,32 @@ __global__ __launch_bounds__(256) void colsum_finalize_kernel(const double *__re
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-template <typename T, int BM, int BN>
-int launch_tile(const MatmulArgs &g, bool ta, bool tb, hipStream_t st)
+template <typename T, int BM, int BN, bool GUARD>
+int launch_tile_guard(const MatmulArgs &g, bool ta, bool tb, hipStream_t st)
 {
     const int64_t tiles = (int64_t)((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
     if (tiles > 0x7fffffff)
         return VTL_HIP_ERR_UNSUPPORTED;
     const dim3 grid((unsigned)tiles), block(256);
     if (!ta && !tb)
-        hipLaunchKernelGGL((matmul_f64acc_kernel<T, BM, BN, false, false>), grid, block, 0, st, g);
+        hipLaunchKernelGGL((matmul_f64acc_kernel<T, BM, BN, false, false, GUARD>), grid, block, 0, st, g);
     else if (!ta && tb)
-        hipLaunchKernelGGL((matmul_f64acc_kernel<T, BM, BN, false, true>), grid, block, 0, st, g);
+        hipLaunchKernelGGL((matmul_f64acc_kernel<T, BM, BN, false, true, GUARD>), grid, block, 0, st, g);
     else if (ta && !tb)
-        hipLaunchKernelGGL((matmul_f64acc_kernel<T, BM, BN, true, false>), grid, block, 0, st, g);
+        hipLaunchKernelGGL((matmul_f64acc_kernel<T, BM, BN, true, false, GUARD>), grid, block, 0, st, g);
     else
-        hipLaunchKernelGGL((matmul_f64acc_kernel<T, BM, BN, true, true>), grid, block, 0, st, g);
+        hipLaunchKernelGGL((matmul_f64acc_kernel<T, BM, BN, true, true, GUARD>), grid, block, 0, st, g);
     return check_launch("matmul_f64acc_kernel");
+}
+
+// Shapes made of whole tiles with 16-byte aligned rows run without bounds checks.
+template <typename T, int BM, int BN>
+int launch_tile(const MatmulArgs &g, bool ta, bool tb, hipStream_t st)
+{
+    const bool whole = g.M % BM == 0 && g.N % BN == 0 && g.K % 16 == 0 && g.K > 0 && g.vec_a && g.vec_b &&
+                       g.vec_c;
+    return whole ? launch_tile_guard<T, BM, BN, false>(g, ta, tb, st)
+                 : launch_tile_guard<T, BM, BN, true>(g, ta, tb, st);
 }
 
 template <typename T>
