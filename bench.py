@@ -30,6 +30,7 @@ from vtl_amd.tensor import HipTensor  # noqa: E402
 METRIC = "int8 Linear TOPS @M=N=K=4096 + quant/dequant GB/s, % of MI355X roofline"
 PEAK_INT8_TOPS = 5000.0      # dense int8 MFMA, MI355X published
 PEAK_HBM_GBPS = 8000.0       # HBM3E, MI355X published
+PEAK_FP64_TFLOPS = 78.6      # dense f64 MFMA, MI355X published
 
 # HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # script, each counter scaled by its reading for the 1 GiB copy_kernel (x2.000 and
@@ -247,6 +248,50 @@ def bench_other_configs(timer: Timer, steps: int, warmup: int):
     return out
 
 
+def bench_full_precision(timer: Timer, steps: int, warmup: int):
+    """The f32 matmul with f64 accumulation behind la.matmul / Linear backward
+    (parity in tests/): the unquantized Linear forward at M=N=K=4096 against the
+    f64 matrix-core peak, and LinearGate.backward of the first MLP layer."""
+    out = {}
+    steps = max(3, min(steps, 10))
+    warmup = max(1, min(warmup, 2))
+    rng = np.random.Generator(np.random.Philox(5))
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        _, dev_ms = timer.run(fn, steps)
+        return dev_ms / steps * 1e3   # microseconds
+
+    m = n = k = 4096
+    X = HipTensor.from_host(rng.standard_normal((m, k), dtype=np.float32))
+    W = HipTensor.from_host(rng.standard_normal((n, k), dtype=np.float32))
+    B = HipTensor.from_host(rng.standard_normal(n, dtype=np.float32))
+    Y = HipTensor.empty([m, n], np.float32)
+    us = timed(lambda: capi.call("vtl_hip_linear_f32", X.ptr, W.ptr, B.ptr, Y.ptr, m, n, k, 0))
+    tf = 2.0 * m * n * k / us / 1e6
+    out["linear_f32 (f64 accumulate) M=N=K=4096"] = {
+        "us": us, "TFLOP/s": tf,
+        "roofline": {"bound": "mfma", "achieved": tf, "peak": PEAK_FP64_TFLOPS, "unit": "TFLOP/s",
+                     "frac": tf / PEAK_FP64_TFLOPS, "traffic": None,
+                     "kernel": "matmul_f64acc_kernel<float, 128, 128, false, true, false>"}}
+    for h in (X, W, B, Y):
+        h.release()
+
+    m, n, k = 256, 11008, 4096
+    G = HipTensor.from_host(rng.standard_normal((m, n), dtype=np.float32))
+    X = HipTensor.from_host(rng.standard_normal((m, k), dtype=np.float32))
+    W = HipTensor.from_host(rng.standard_normal((n, k), dtype=np.float32))
+    dX, dW, dB = HipTensor.empty([m, k], np.float32), HipTensor.empty([n, k], np.float32), HipTensor.empty([n], np.float32)
+    us = timed(lambda: capi.call("vtl_hip_linear_backward_f32", G.ptr, X.ptr, W.ptr, dX.ptr, dW.ptr, dB.ptr, m, n, k))
+    out["linear_backward_f32 grad[256,11008] x[256,4096] W[11008,4096] (dx, dw, db)"] = {
+        "us": us, "TFLOP/s": 4.0 * m * n * k / us / 1e6, "frac_of_fp64_mfma_peak": 4.0 * m * n * k / us / 1e6 / PEAK_FP64_TFLOPS}
+    capi.call("vtl_hip_sync")
+    for h in (G, X, W, dX, dW, dB):
+        h.release()
+    return out
+
+
 def bench_copy_calibration(timer: Timer, steps: int, warmup: int):
     """Plain device-to-device copy of 1 GiB with the library's copy kernel: the
     kernel of known traffic (1 GiB read + 1 GiB written per launch) that the
@@ -323,6 +368,7 @@ def main() -> int:
         line["dequantize"] = qd["dequantize"]
     if args.only == "all":
         line["other_configs"] = bench_other_configs(timer, args.steps, args.warmup)
+        line["full_precision"] = bench_full_precision(timer, args.steps, args.warmup)
     print(json.dumps(line))
     return 0
 
