@@ -119,6 +119,36 @@ int main(int argc, char **argv)
         } catch (const std::invalid_argument &) {
         }
     }
+    // la.matmul and LinearGate.backward with f64 accumulation vs oracle: integer-valued
+    // operands, for which every summation order gives the same bits
+    {
+        std::uniform_int_distribution<int> ud(-8, 8);
+        std::vector<float> g((size_t)M * N), xi((size_t)M * K), wi((size_t)N * K);
+        for (auto &v : g) v = (float)ud(rng);
+        for (auto &v : xi) v = (float)ud(rng);
+        for (auto &v : wi) v = (float)ud(rng);
+        auto G = vtl::HipTensor<float>::from_host(g, {M, N});
+        auto W = vtl::HipTensor<float>::from_host(wi, {N, K});
+        auto X = vtl::HipTensor<float>::from_host(xi, {M, K});
+        std::vector<float> ref((size_t)M * K);
+        vtl_ref_matmul_f32(g.data(), wi.data(), ref.data(), M, K, N, 0, 0, 1);
+        CHECK(vtl::matmul_hip(G, W).cpu() == ref);                 // grad . W
+        std::vector<float> ref_t((size_t)N * K);
+        vtl_ref_matmul_f32(g.data(), xi.data(), ref_t.data(), N, K, M, 1, 0, 1);
+        CHECK(vtl::matmul_hip(G, X, true, false).cpu() == ref_t);  // grad^T . x
+        try {
+            vtl::matmul_hip(G, X);
+            CHECK(false);
+        } catch (const std::invalid_argument &e) {
+            CHECK(std::strstr(e.what(), "Invalid shapes for matrix multiplication"));
+        }
+        std::vector<float> dx((size_t)M * K), dw((size_t)N * K), db(N);
+        vtl_ref_linear_backward_f32(g.data(), xi.data(), wi.data(), dx.data(), dw.data(), db.data(), M, N, K, 1);
+        auto got = vtl::linear_backward_hip_f32(g, M, N, xi, K, wi, true);
+        CHECK(got[0] == dx && got[1] == dw && got[2] == db);
+        auto no_bias = vtl::linear_backward_hip_f32(g, M, N, xi, K, wi, false);
+        CHECK(no_bias[0] == dx && no_bias[2] == std::vector<float>(N, 0.0f));
+    }
     std::printf(failures ? "host mirror: %d failure(s)\n" : "host mirror: ok\n", failures);
     return failures ? 1 : 0;
 }

@@ -233,4 +233,54 @@ inline std::vector<float> linear_forward_hip_f32(const std::vector<float> &x, in
     return y.cpu();
 }
 
+// `matmul_hip(a, b, trans_a, trans_b) !&HipTensor[T]`: la.matmul (la/la.v:38-55)
+// on the device, f64 products and sums, one rounding to T (float or double).
+template <typename T>
+inline HipTensor<T> matmul_hip(const HipTensor<T> &a, const HipTensor<T> &b, bool trans_a = false,
+                               bool trans_b = false)
+{
+    static_assert(std::is_same<T, float>::value || std::is_same<T, double>::value, "f32 or f64");
+    if (!a.is_matrix() || !b.is_matrix())
+        throw std::invalid_argument("Matrix expected");
+    const int m = trans_a ? a.shape[1] : a.shape[0], k = trans_a ? a.shape[0] : a.shape[1];
+    const int k2 = trans_b ? b.shape[1] : b.shape[0], n = trans_b ? b.shape[0] : b.shape[1];
+    if (k != k2)
+        throw std::invalid_argument("Invalid shapes for matrix multiplication");
+    HipTensor<T> c({m, n}, HipParams{a.data.device_id});
+    if (std::is_same<T, float>::value)
+        hip_check(vtl_hip_matmul_f32((const float *)a.data.ptr, (const float *)b.data.ptr, (float *)c.data.ptr, m,
+                                     n, k, trans_a, trans_b),
+                  "vtl_hip_matmul_f32");
+    else
+        hip_check(vtl_hip_matmul_f64((const double *)a.data.ptr, (const double *)b.data.ptr,
+                                     (double *)c.data.ptr, m, n, k, trans_a, trans_b),
+                  "vtl_hip_matmul_f64");
+    return c;
+}
+
+// `linear_backward_hip_f32(grad, input, weight, bias_needs_grad) ![]&vtl.Tensor[f32]`
+// (cf. linear_backward_vulkan_f32, nn/internal/linear_vulkan_backward_d_vulkan.v:9-38):
+// host tensors in, {d_input[M,K], d_weight[N,K], d_bias[1,N]} out; d_bias is zeros
+// when the bias needs no gradient.
+inline std::vector<std::vector<float>> linear_backward_hip_f32(const std::vector<float> &grad, int m, int n,
+                                                               const std::vector<float> &input, int k,
+                                                               const std::vector<float> &weight,
+                                                               bool bias_needs_grad)
+{
+    if (grad.size() != (size_t)m * n || input.size() != (size_t)m * k || weight.size() != (size_t)n * k)
+        throw std::invalid_argument("linear_backward_hip_f32: shapes of grad, input and weight disagree");
+    auto g_dev = HipTensor<float>::from_host(grad, {m, n});
+    auto x_dev = HipTensor<float>::from_host(input, {m, k});
+    auto w_dev = HipTensor<float>::from_host(weight, {n, k});
+    HipTensor<float> dx({m, k}), dw({n, k});
+    HipStorage<float> db;
+    if (bias_needs_grad)
+        db = HipStorage<float>((size_t)n);
+    hip_check(vtl_hip_linear_backward_f32((const float *)g_dev.data.ptr, (const float *)x_dev.data.ptr,
+                                          (const float *)w_dev.data.ptr, (float *)dx.data.ptr,
+                                          (float *)dw.data.ptr, (float *)db.ptr, m, n, k),
+              "vtl_hip_linear_backward_f32");
+    return {dx.cpu(), dw.cpu(), bias_needs_grad ? db.to_array() : std::vector<float>((size_t)n, 0.0f)};
+}
+
 }  // namespace vtl
