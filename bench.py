@@ -274,7 +274,7 @@ def bench_full_precision(timer: Timer, steps: int, warmup: int):
         "us": us, "TFLOP/s": tf,
         "roofline": {"bound": "mfma", "achieved": tf, "peak": PEAK_FP64_TFLOPS, "unit": "TFLOP/s",
                      "frac": tf / PEAK_FP64_TFLOPS, "traffic": None,
-                     "kernel": "matmul_f64acc_kernel<float, 128, 128, false, true, false>"}}
+                     "kernel": "matmul_f64acc_kernel<float, 128, 128, false, true, false, false>"}}
     for h in (X, W, B, Y):
         h.release()
 
@@ -320,7 +320,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["all", "linear", "quant", "copy"], default="all")
+    ap.add_argument("--only", choices=["all", "linear", "quant", "copy", "full"], default="all")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 "
@@ -335,6 +335,9 @@ def main() -> int:
     cpu = not args.no_cpu_baseline
     if args.only == "copy":
         print(json.dumps({"calibration": bench_copy_calibration(timer, args.steps, args.warmup)}))
+        return 0
+    if args.only == "full":
+        print(json.dumps({"full_precision": bench_full_precision(timer, args.steps, args.warmup)}))
         return 0
 
     lin = bench_linear(timer, args.steps, args.warmup, cpu) if args.only in ("all", "linear") else None

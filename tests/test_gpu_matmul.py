@@ -65,6 +65,44 @@ def test_matmul_shapes_and_layouts(hip, dt, ta, tb):
         assert_close_to_oracle(got, want, absprod)
 
 
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_split_k_paths(hip, dt, monkeypatch):
+    """Few output tiles and a long K slice K over the grid; forced slice counts cover
+    ragged K, edge tiles and the unsplit fallback."""
+    rng = np.random.default_rng(27)
+    cases = [(256, 4096, 11008, False, False, None), (256, 1024, 4096, False, True, None),
+             (64, 64, 2048, True, False, None), (100, 70, 1000, False, True, "3"), (128, 192, 4096, True, True, "5"),
+             (33, 65, 777, False, False, "16"), (64, 128, 96, False, True, "4")]
+    for (M, N, K, ta, tb, force) in cases:
+        if force is None:
+            monkeypatch.delenv("VTL_HIP_MATMUL_SPLITS", raising=False)
+        else:
+            monkeypatch.setenv("VTL_HIP_MATMUL_SPLITS", force)
+        A = rng.standard_normal((K, M) if ta else (M, K)).astype(dt)
+        B = rng.standard_normal((N, K) if tb else (K, N)).astype(dt)
+        print("split-K", dt.__name__, M, N, K, ta, tb, force, flush=True)
+        got = run_matmul(A, B, ta, tb)
+        want = oracle.matmul(A, B, ta, tb, threads=CPU_THREADS)
+        absprod = np.abs(A.T if ta else A).astype(np.float64) @ np.abs(B.T if tb else B).astype(np.float64)
+        assert_close_to_oracle(got, want, absprod)
+        # integer-valued operands: bit for bit whatever the slicing
+        Ai, Bi = np.rint(A * 4).astype(dt), np.rint(B * 4).astype(dt)
+        exact = (Ai.T if ta else Ai).astype(np.float64) @ (Bi.T if tb else Bi).astype(np.float64)
+        assert np.array_equal(run_matmul(Ai, Bi, ta, tb), exact.astype(dt))
+    # the Linear form keeps bias and ReLU after the sliced sum
+    monkeypatch.delenv("VTL_HIP_MATMUL_SPLITS", raising=False)
+    x = rng.standard_normal((128, 4096)).astype(dt)
+    w = (rng.standard_normal((256, 4096)) * 0.05).astype(dt)
+    b = rng.standard_normal(256).astype(dt)
+    xd, wd, bd = dev(x), dev(w), dev(b.reshape(1, -1))
+    y = linear_hip(xd, wd, bd, relu=True)
+    ref = oracle.matmul(x, w, False, True) + b
+    assert_close_to_oracle(y.cpu(), np.where(ref < 0, dt(0), ref).astype(dt),
+                           np.abs(x).astype(np.float64) @ np.abs(w.T).astype(np.float64) + np.abs(b))
+    for t in (xd, wd, bd, y):
+        t.release()
+
+
 def test_reference_literals(hip):
     # la/la_test.v:30-37
     a = np.array([[1.0, 0], [0.0, 1]])

@@ -13,6 +13,8 @@
 // columns), which makes those reads and the final stores contiguous per lane.
 #include "common.hpp"
 
+#include <stdlib.h>
+
 #include <type_traits>
 
 namespace {
@@ -30,6 +32,8 @@ struct MatmulArgs {
     int M, N, K;
     int vec_a, vec_b, vec_c;   // base 16-byte aligned and leading dimension % 4 == 0
     int relu;
+    int k_per_split;           // split-K launches: k range of one grid.y slice (multiple of 16)
+    double *partial;           // split-K launches: [splits][M][N] unrounded sums
 };
 
 template <typename T>
@@ -78,8 +82,10 @@ struct OperandTile {
     static_assert(kGroups % 256 == 0 || kGroups == 128, "tile must split over 256 threads");
     Vec4<T> regs[kPerThread];
 
-    __device__ __forceinline__ void fetch(const T *__restrict__ base, int mn_total, int k_total, int mn0,
-                                          int k0, bool vec_ok)
+    // k_total: the matrix's K (its leading dimension when stored [MN, K]);
+    // k_limit <= k_total: positions with k >= k_limit read as zero.
+    __device__ __forceinline__ void fetch(const T *__restrict__ base, int mn_total, int k_total, int k_limit,
+                                          int mn0, int k0, bool vec_ok)
     {
         const int t = threadIdx.x;
 #pragma unroll
@@ -89,10 +95,10 @@ struct OperandTile {
                 break;
             if constexpr (KMAJOR) {
                 const int krow = g / (BMN / 4), c4 = g % (BMN / 4);
-                regs[i] = load4<T, GUARD>(base, mn_total, k_total, mn_total, k0 + krow, mn0 + 4 * c4, vec_ok);
+                regs[i] = load4<T, GUARD>(base, mn_total, k_limit, mn_total, k0 + krow, mn0 + 4 * c4, vec_ok);
             } else {
                 const int mn = g % BMN, kc = g / BMN;
-                regs[i] = load4<T, GUARD>(base, k_total, mn_total, k_total, mn0 + mn, k0 + 4 * kc, vec_ok);
+                regs[i] = load4<T, GUARD>(base, k_total, mn_total, k_limit, mn0 + mn, k0 + 4 * kc, vec_ok);
             }
         }
     }
@@ -120,7 +126,8 @@ struct OperandTile {
 
 // GUARD == false: M, N, K are whole tiles and every row is 16-byte aligned, so
 // the loads and stores carry no bounds checks and the k-loop is straight-line code.
-template <typename T, int BM, int BN, bool TA, bool TB, bool GUARD>
+// SPLIT: grid.y slices K; each slice writes its unrounded f64 sums to g.partial.
+template <typename T, int BM, int BN, bool TA, bool TB, bool GUARD, bool SPLIT>
 __global__ __launch_bounds__(256) void matmul_f64acc_kernel(const MatmulArgs g)
 {
     constexpr int BK = 64 / (int)sizeof(T);   // 16 for f32, 8 for f64
@@ -153,9 +160,11 @@ __global__ __launch_bounds__(256) void matmul_f64acc_kernel(const MatmulArgs g)
         for (int j = 0; j < TN; ++j)
             acc[i][j] = double4_t{0.0, 0.0, 0.0, 0.0};
 
-    const int ktiles = (g.K + BK - 1) / BK;
-    ta.fetch(A, g.M, g.K, m0, 0, g.vec_a != 0);
-    tb.fetch(B, g.N, g.K, n0, 0, g.vec_b != 0);
+    const int k_begin = SPLIT ? (int)blockIdx.y * g.k_per_split : 0;
+    const int k_end = SPLIT ? (k_begin + g.k_per_split < g.K ? k_begin + g.k_per_split : g.K) : g.K;
+    const int ktiles = (k_end - k_begin + BK - 1) / BK;
+    ta.fetch(A, g.M, g.K, k_end, m0, k_begin, g.vec_a != 0);
+    tb.fetch(B, g.N, g.K, k_end, n0, k_begin, g.vec_b != 0);
     ta.stash(As[0]);
     tb.stash(Bs[0]);
     __syncthreads();
@@ -163,8 +172,8 @@ __global__ __launch_bounds__(256) void matmul_f64acc_kernel(const MatmulArgs g)
     for (int kt = 0; kt < ktiles; ++kt) {
         const int cur = kt & 1;
         if (kt + 1 < ktiles) {
-            ta.fetch(A, g.M, g.K, m0, (kt + 1) * BK, g.vec_a != 0);
-            tb.fetch(B, g.N, g.K, n0, (kt + 1) * BK, g.vec_b != 0);
+            ta.fetch(A, g.M, g.K, k_end, m0, k_begin + (kt + 1) * BK, g.vec_a != 0);
+            tb.fetch(B, g.N, g.K, k_end, n0, k_begin + (kt + 1) * BK, g.vec_b != 0);
         }
         const T *__restrict__ as = As[cur] + wm + TM * r16;
         const T *__restrict__ bs = Bs[cur] + wn + TN * r16;
@@ -191,6 +200,21 @@ __global__ __launch_bounds__(256) void matmul_f64acc_kernel(const MatmulArgs g)
     // Element e of MFMA tile (i, j) in lane l is row 4 * e + l / 16, column
     // l % 16 of that tile (the f64 16x16x4 layout): matrix row
     // wm + TM * (4 * e + kq) + i, columns wn + TN * r16 + j (j contiguous).
+    if constexpr (SPLIT) {
+        double *__restrict__ P = g.partial + (int64_t)blockIdx.y * g.M * g.N;
+        const int pcol0 = n0 + wn + TN * r16;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int row = m0 + wm + TM * (4 * e + kq) + i;
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    if (!GUARD || (row < g.M && pcol0 + j < g.N))
+                        P[(int64_t)row * g.N + pcol0 + j] = acc[i][j][e];
+            }
+        return;
+    }
     T *__restrict__ C = static_cast<T *>(g.C);
     const T *__restrict__ bias = static_cast<const T *>(g.bias);
     const int col0 = n0 + wn + TN * r16;
@@ -316,23 +340,44 @@ __global__ __launch_bounds__(256) void colsum_finalize_kernel(const double *__re
     out[c] = (T)s;
 }
 
+// Sums the K slices of a split launch in slice order, rounds once to T, then
+// bias and ReLU as in the unsplit epilogue.
+template <typename T>
+__global__ __launch_bounds__(256) void matmul_splitk_finalize_kernel(const MatmulArgs g, int splits)
+{
+    const int64_t total = (int64_t)g.M * g.N;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total)
+        return;
+    double s = 0.0;
+    for (int i = 0; i < splits; ++i)
+        s += g.partial[(int64_t)i * total + idx];
+    T y = (T)s;
+    const T *__restrict__ bias = static_cast<const T *>(g.bias);
+    if (bias)
+        y = y + bias[idx % g.N];
+    if (g.relu && y < T(0))
+        y = T(0);
+    static_cast<T *>(g.C)[idx] = y;
+}
+
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-template <typename T, int BM, int BN, bool GUARD>
-int launch_tile_guard(const MatmulArgs &g, bool ta, bool tb, hipStream_t st)
+template <typename T, int BM, int BN, bool GUARD, bool SPLIT>
+int launch_tile_guard(const MatmulArgs &g, bool ta, bool tb, int splits, hipStream_t st)
 {
     const int64_t tiles = (int64_t)((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
     if (tiles > 0x7fffffff)
         return VTL_HIP_ERR_UNSUPPORTED;
-    const dim3 grid((unsigned)tiles), block(256);
+    const dim3 grid((unsigned)tiles, (unsigned)splits), block(256);
     if (!ta && !tb)
-        hipLaunchKernelGGL((matmul_f64acc_kernel<T, BM, BN, false, false, GUARD>), grid, block, 0, st, g);
+        hipLaunchKernelGGL((matmul_f64acc_kernel<T, BM, BN, false, false, GUARD, SPLIT>), grid, block, 0, st, g);
     else if (!ta && tb)
-        hipLaunchKernelGGL((matmul_f64acc_kernel<T, BM, BN, false, true, GUARD>), grid, block, 0, st, g);
+        hipLaunchKernelGGL((matmul_f64acc_kernel<T, BM, BN, false, true, GUARD, SPLIT>), grid, block, 0, st, g);
     else if (ta && !tb)
-        hipLaunchKernelGGL((matmul_f64acc_kernel<T, BM, BN, true, false, GUARD>), grid, block, 0, st, g);
+        hipLaunchKernelGGL((matmul_f64acc_kernel<T, BM, BN, true, false, GUARD, SPLIT>), grid, block, 0, st, g);
     else
-        hipLaunchKernelGGL((matmul_f64acc_kernel<T, BM, BN, true, true, GUARD>), grid, block, 0, st, g);
+        hipLaunchKernelGGL((matmul_f64acc_kernel<T, BM, BN, true, true, GUARD, SPLIT>), grid, block, 0, st, g);
     return check_launch("matmul_f64acc_kernel");
 }
 
@@ -342,8 +387,31 @@ int launch_tile(const MatmulArgs &g, bool ta, bool tb, hipStream_t st)
 {
     const bool whole = g.M % BM == 0 && g.N % BN == 0 && g.K % 16 == 0 && g.K > 0 && g.vec_a && g.vec_b &&
                        g.vec_c;
-    return whole ? launch_tile_guard<T, BM, BN, false>(g, ta, tb, st)
-                 : launch_tile_guard<T, BM, BN, true>(g, ta, tb, st);
+    return whole ? launch_tile_guard<T, BM, BN, false, false>(g, ta, tb, 1, st)
+                 : launch_tile_guard<T, BM, BN, true, false>(g, ta, tb, 1, st);
+}
+
+// Few output tiles and a long K: slice K over grid.y so that every SIMD holds
+// several waves, f64 partial sums in the library's workspace, then one pass
+// that adds the slices in order and rounds.
+template <typename T>
+int launch_split(MatmulArgs g, bool ta, bool tb, int splits, hipStream_t st)
+{
+    const int per = ((g.K + splits - 1) / splits + 15) / 16 * 16;
+    splits = (g.K + per - 1) / per;
+    g.k_per_split = per;
+    g.partial = static_cast<double *>(
+        vtlhip::library_workspace((size_t)splits * (size_t)g.M * (size_t)g.N * sizeof(double)));
+    if (!g.partial)
+        return VTL_HIP_ERR_OUT_OF_MEMORY;
+    const bool whole = g.M % 64 == 0 && g.N % 64 == 0 && g.K % per == 0 && g.vec_a && g.vec_b;
+    int rc = whole ? launch_tile_guard<T, 64, 64, false, true>(g, ta, tb, splits, st)
+                   : launch_tile_guard<T, 64, 64, true, true>(g, ta, tb, splits, st);
+    if (rc != VTL_HIP_OK)
+        return rc;
+    const int64_t blocks = ((int64_t)g.M * g.N + 255) / 256;
+    hipLaunchKernelGGL((matmul_splitk_finalize_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, st, g, splits);
+    return check_launch("matmul_splitk_finalize_kernel");
 }
 
 template <typename T>
@@ -369,11 +437,25 @@ int matmul_impl(const T *a, const T *b, T *c, const T *bias, int m, int n, int k
     g.vec_b = aligned16(b) && ldb % 4 == 0;
     g.vec_c = aligned16(c) && n % 4 == 0;
     g.relu = relu;
+    g.k_per_split = 0;
+    g.partial = nullptr;
     hipStream_t st = current_stream();
     // 128x128 tiles once they fill the 256 compute units; 64x64 tiles otherwise
     const int64_t big = (int64_t)((m + 127) / 128) * ((n + 127) / 128);
     if (big >= 192)
         return launch_tile<T, 128, 128>(g, trans_a != 0, trans_b != 0, st);
+    const int64_t small = (int64_t)((m + 63) / 64) * ((n + 63) / 64);
+    const char *force = getenv("VTL_HIP_MATMUL_SPLITS");   // tuning and tests
+    int splits = force ? atoi(force) : 1;
+    if (!force && small <= 512 && k >= 2048) {
+        splits = (int)(1024 / small);
+        if (splits > k / 512)
+            splits = k / 512;
+        if (splits > 16)
+            splits = 16;
+    }
+    if (splits > 1 && k >= 32 * splits)
+        return launch_split<T>(g, trans_a != 0, trans_b != 0, splits, st);
     return launch_tile<T, 64, 64>(g, trans_a != 0, trans_b != 0, st);
 }
 
