@@ -145,6 +145,32 @@ ROUTED_SHAPES = [(1, 2048, 256), (3, 2050, 256), (8, 2048, 4096), (9, 2048, 768)
                  (17, 2077, 1280), (32, 4096, 512), (31, 14336, 256), (5, 3001, 4096),
                  (256, 1024, 4096), (256, 512, 11008), (64, 128, 11008), (128, 256, 8192), (40, 200, 5504),
                  (100, 300, 1360), (256, 256, 1040)]
+# small products: one 32x32 tile per workgroup fed straight from global memory
+# (at most 64 tiles, K <= 2048), incl. K % 32 == 16, single rows and columns
+SMALL_SHAPES = [(64, 256, 784), (1, 1, 16), (2, 3, 16), (33, 65, 48), (64, 64, 2048), (31, 1, 1008),
+                (1, 97, 2032), (256, 256, 512), (100, 300, 1360), (256, 256, 1040)]
+
+
+@pytest.mark.parametrize("small", ["0", "1", None])
+@pytest.mark.parametrize("mnk", SMALL_SHAPES)
+def test_small_product_kernel_and_its_alternatives(hip, mnk, small, monkeypatch):
+    """VTL_HIP_GEMM_SMALL=1 forces the small-product kernel, 0 the tile kernels the
+    same shapes used before it existed, unset the library's own choice."""
+    if small is None:
+        monkeypatch.delenv("VTL_HIP_GEMM_SMALL", raising=False)
+    else:
+        monkeypatch.setenv("VTL_HIP_GEMM_SMALL", small)
+    m, n, k = mnk
+    a, bt, sa, sb, bias = workloads.square_int8_gemm(m, n, k, seed=m * 17 + n * 5 + k)
+    ref = oracle.gemm_i8_i32(a, bt, threads=CPU_THREADS)
+    assert np.array_equal(_gemm(a, bt), ref)
+    A, B, dsa, dsb, dbias = dev(a), dev(bt), dev(sa), dev(sb), dev(bias)
+    for relu, b_dev, b_host in ((True, dbias, bias), (False, None, None)):
+        y = linear_i8_hip(A, dsa, B, dsb, b_dev, relu=relu)
+        assert np.array_equal(y.cpu(), oracle.epilogue(ref, sa, sb, b_host, relu=relu))
+        y.release()
+    for h in (A, B, dsa, dsb, dbias):
+        h.release()
 
 
 @pytest.mark.parametrize("mnk", ROUTED_SHAPES)

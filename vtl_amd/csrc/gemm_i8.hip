@@ -873,6 +873,73 @@ __global__ __launch_bounds__(256) void gemm_i8_naive_kernel(const GemmArgs g)
     }
 }
 
+// Small products (a few dozen 32x32 output tiles): nothing is reused often
+// enough to stage, so each wave feeds the MFMA straight from global memory.
+// One workgroup per 32x32 tile; its four waves split the K steps and the
+// partial tiles meet in LDS.  Needs K % 16 == 0 and 16-byte aligned operands.
+template <bool F32OUT>
+__global__ __launch_bounds__(256) void gemm_i8_small_kernel(const GemmArgs g)
+{
+    __shared__ int red[4][16][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int tiles_n = (g.N + 31) / 32;
+    const int m0 = (int)(blockIdx.x / tiles_n) * 32, n0 = (int)(blockIdx.x % tiles_n) * 32;
+    const int r = lane & 31, half = lane >> 5;
+    // rows past the edge repeat the last row; their results are never stored
+    const int arow = m0 + r < g.M ? m0 + r : g.M - 1;
+    const int brow = n0 + r < g.N ? n0 + r : g.N - 1;
+    const int8_t *__restrict__ ap = g.A + (int64_t)arow * g.K + 16 * half;
+    const int8_t *__restrict__ bp = g.Bt + (int64_t)brow * g.K + 16 * half;
+    const int steps = (g.K + 31) / 32;
+    const int per = (steps + 3) / 4;
+    const int t0 = wave * per, t1 = t0 + per < steps ? t0 + per : steps;
+    v16i acc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+        acc[i] = 0;
+    const v4i zero = {0, 0, 0, 0};
+    for (int t = t0; t < t1; t += 4) {   // four steps of loads in flight
+        v4i a[4], b[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int k = 32 * (t + u);
+            // K % 32 == 16: the upper half of the last step is empty
+            const bool in = t + u < t1 && k + 16 * half < g.K;
+            a[u] = in ? *reinterpret_cast<const v4i *>(ap + k) : zero;
+            b[u] = in ? *reinterpret_cast<const v4i *>(bp + k) : zero;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[u], b[u], acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+        red[wave][i][lane] = acc[i];
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int o = threadIdx.x + 256 * j;
+        const int reg = o >> 6, l = o & 63;
+        const int sum = (red[0][reg][l] + red[1][reg][l]) + (red[2][reg][l] + red[3][reg][l]);
+        // accumulator register reg of lane l: row 8 * (reg / 4) + 4 * (l / 32) + reg % 4, column l % 32
+        const int m = m0 + 8 * (reg >> 2) + 4 * (l >> 5) + (reg & 3), n = n0 + (l & 31);
+        if (m >= g.M || n >= g.N)
+            continue;
+        const int64_t idx = (int64_t)m * g.N + n;
+        if (F32OUT) {
+            const float sc = g.sa[(int64_t)m * g.sa_stride] * g.sw[(int64_t)n * g.sw_stride];
+            float y = (float)sum * sc;
+            if (g.bias)
+                y = y + g.bias[n];
+            if (g.relu && y < 0.0f)
+                y = 0.0f;
+            reinterpret_cast<float *>(g.out)[idx] = y;
+        } else {
+            reinterpret_cast<int32_t *>(g.out)[idx] = sum;
+        }
+    }
+}
+
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 template <typename Kern>
@@ -1050,6 +1117,12 @@ int launch_gemm(const GemmArgs &g, hipStream_t st)
     }
     if (g.K % 256 == 0 && g.M <= 32 && g.N >= 2048 && !getenv("VTL_HIP_GEMM_CONFIG"))
         return launch_skinny<F32OUT>(g, st);  // weight streaming: enough row blocks to fill the chip
+    const int64_t t32 = (int64_t)((g.M + 31) / 32) * ((g.N + 31) / 32);
+    const char *small_env = getenv("VTL_HIP_GEMM_SMALL");   // "1" / "0" force the choice (tests, tuning)
+    if (small_env ? atoi(small_env) != 0 : (t32 <= 64 && g.K <= 2048)) {
+        hipLaunchKernelGGL((gemm_i8_small_kernel<F32OUT>), dim3((unsigned)t32), dim3(256), 0, st, g);
+        return check_launch("gemm_i8_small_kernel");
+    }
     if (g.K % 128 == 0) {
         int idx, splits;
         choose_config(g.M, g.N, g.K, idx, splits);

@@ -474,6 +474,11 @@ int vtl_hip_quantize_f32_i8(const float *x, int64_t rows, int64_t cols, int per_
     hipStream_t s = current_stream();
     if (per_row)
         return launch_quantize_rows(x, rows, cols, q, scale_out, s);
+    // a small tensor is one "row" of the fused kernel: a single workgroup holds it
+    // in registers between the absmax and the rounding pass, one launch instead of four
+    const int64_t total = rows * cols;
+    if (total > 0 && total <= 4 * 1024 * 16 && total % 4 == 0 && aligned(x, 16) && aligned(q, 4))
+        return launch_quantize_rows(x, 1, total, q, scale_out, s);
     // whole tensor: absmax pass, scale in place, then the scaled quantize pass
     st = vtl_hip_absmax_f32(x, rows, cols, 0, scale_out);
     if (st != VTL_HIP_OK)
