@@ -1,0 +1,106 @@
+"""Tensors with more than 2^31 elements: every kernel indexes with 64 bits.
+The inputs are a random block repeated many times plus a few planted values
+at the far end, so the oracle only has to restate one block and the planted
+rows; the whole device result is compared."""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import CPU_THREADS, dev
+from vtl_amd import capi
+from vtl_amd.tensor import HipTensor, linear_i8_hip
+
+pytestmark = pytest.mark.gpu
+
+BLOCK_ROWS, REPS, EXTRA, COLS = 4096, 256, 3, 2052      # (4096 * 256 + 3) * 2052 = 2 151 683 100 > 2^31
+
+
+def _big_input():
+    rng = np.random.default_rng(31)
+    block = rng.standard_normal((BLOCK_ROWS, COLS)).astype(np.float32)
+    rows = BLOCK_ROWS * REPS + EXTRA
+    x = np.empty((rows, COLS), np.float32)
+    x[: BLOCK_ROWS * REPS].reshape(REPS, BLOCK_ROWS, COLS)[:] = block
+    x[BLOCK_ROWS * REPS:] = block[:EXTRA]
+    x[-1, -1] = np.float32(1000.0)          # the very last element carries the tensor's absmax
+    x[-2, 0] = np.float32(-77.0)
+    return block, x
+
+
+def test_quantize_dequantize_beyond_2_31_elements(hip):
+    block, x = _big_input()
+    rows = x.shape[0]
+    assert x.size > 2 ** 31
+    print("upload", x.nbytes >> 20, "MiB", flush=True)
+    X = dev(x)
+    tail = x[BLOCK_ROWS * REPS:]
+
+    # one scale per row: rows are independent, so the block's codes repeat
+    print("per-row quantize", flush=True)
+    Q, S = X.quantize_i8(0)
+    q, s = Q.cpu(), S.cpu().reshape(-1)
+    qb, sb = oracle.quantize(block, True, threads=CPU_THREADS)
+    qt, st = oracle.quantize(tail, True)
+    assert np.array_equal(s[: BLOCK_ROWS * REPS].reshape(REPS, BLOCK_ROWS), np.broadcast_to(sb, (REPS, BLOCK_ROWS)))
+    assert np.array_equal(q[: BLOCK_ROWS * REPS].reshape(REPS, BLOCK_ROWS, COLS),
+                          np.broadcast_to(qb, (REPS, BLOCK_ROWS, COLS)))
+    assert np.array_equal(q[BLOCK_ROWS * REPS:], qt) and np.array_equal(s[BLOCK_ROWS * REPS:], st)
+    assert q[-1, -1] == 127 and s[-1] == np.float32(1000.0) / np.float32(127.0)
+
+    print("per-row dequantize", flush=True)
+    D = Q.dequantize(S, 0)
+    d = D.cpu()
+    db = oracle.dequantize(qb, sb, True)
+    assert np.array_equal(d[: BLOCK_ROWS * REPS].reshape(REPS, BLOCK_ROWS, COLS),
+                          np.broadcast_to(db, (REPS, BLOCK_ROWS, COLS)))
+    assert np.array_equal(d[BLOCK_ROWS * REPS:], oracle.dequantize(qt, st, True))
+    for h in (Q, S, D):
+        h.release()
+    del q, d
+
+    # one scale for the tensor: the planted last element sets it
+    print("per-tensor quantize", flush=True)
+    A = X.absmax(-1)
+    assert A.cpu()[0] == np.float32(1000.0)
+    Q, S = X.quantize_i8(-1)
+    scale = S.cpu().reshape(-1)
+    assert scale[0] == np.float32(1000.0) / np.float32(127.0)
+    q = Q.cpu()
+    qb = oracle.quantize_with_scale(block, scale, False)
+    assert np.array_equal(q[: BLOCK_ROWS * REPS].reshape(REPS, BLOCK_ROWS, COLS),
+                          np.broadcast_to(qb, (REPS, BLOCK_ROWS, COLS)))
+    assert np.array_equal(q[BLOCK_ROWS * REPS:], oracle.quantize_with_scale(tail, scale, False))
+    assert q[-1, -1] == 127 and q[-2, 0] == -10      # -77 / (1000/127) = -9.779 -> -10
+    for h in (X, A, Q, S):
+        h.release()
+
+
+def test_linear_output_beyond_2_31_elements(hip):
+    """[46400, 128] x [46400, 128]^T: 2.15e9 outputs; sampled row bands against the oracle."""
+    m = n = 46400
+    k = 128
+    rng = np.random.default_rng(32)
+    a = rng.integers(-127, 128, (m, k), dtype=np.int8)
+    w = rng.integers(-127, 128, (n, k), dtype=np.int8)
+    sa = rng.uniform(0.5, 1.5, m).astype(np.float32)
+    sw = rng.uniform(0.5, 1.5, n).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    assert m * n > 2 ** 31
+    A, W, SA, SW, B = dev(a), dev(w), dev(sa), dev(sw), dev(bias)
+    print("linear", m, n, k, flush=True)
+    Y = linear_i8_hip(A, SA, W, SW, B, relu=True)
+    rows = np.r_[0:8, 23195:23205, m - 8:m]
+    for r0 in (0, 23195, m - 8):
+        band = slice(r0, r0 + 8)
+        got = np.empty((8, n), np.float32)
+        capi.call("vtl_hip_memcpy_d2h", got.ctypes.data, Y.ptr + r0 * n * 4, got.nbytes)
+        want = oracle.linear_i8_f32(a[band], sa[band], w, sw, bias, relu=True, threads=CPU_THREADS)
+        assert np.array_equal(got, want), f"rows {r0}..{r0 + 8}"
+    C = HipTensor.empty([m, n], np.int32)
+    capi.call("vtl_hip_gemm_i8_i32", A.ptr, W.ptr, C.ptr, m, n, k)
+    got = np.empty((8, n), np.int32)
+    capi.call("vtl_hip_memcpy_d2h", got.ctypes.data, C.ptr + (m - 8) * n * 4, got.nbytes)
+    assert np.array_equal(got, oracle.gemm_i8_i32(a[m - 8:], w, threads=CPU_THREADS))
+    del rows
+    for h in (A, W, SA, SW, B, Y, C):
+        h.release()
