@@ -175,6 +175,20 @@ int vtl_hip_linear_backward_f64(const double *grad, const double *x, const doubl
 /* ReLU in place on the device (nn/internal/activation.v:63-70,
  * relu_cuda tensor_cuda_d_cuda.v:205-235). */
 int vtl_hip_relu_f32(float *x, int64_t n);
+int vtl_hip_relu_f64(double *x, int64_t n);
+
+/* ---- generic tensor operations (tensor_cuda_d_cuda.v:182-270) -------------- */
+
+/* y[rows] = A[rows, cols] . x[cols], products and sums in f64, one rounding to
+ * the tensor's type (gemv_cuda, tensor_cuda_d_cuda.v:182-203). */
+int vtl_hip_gemv_f32(const float *A, const float *x, float *y, int64_t rows, int64_t cols);
+int vtl_hip_gemv_f64(const double *A, const double *x, double *y, int64_t rows, int64_t cols);
+
+/* y = 1 / (1 + T(exp(-f64(x)))), the sum and the quotient in the tensor's type
+ * (nn/internal/activation.v:35-40; sigmoid_cuda tensor_cuda_d_cuda.v:237-270).
+ * y may be x. */
+int vtl_hip_sigmoid_f32(const float *x, float *y, int64_t n);
+int vtl_hip_sigmoid_f64(const double *x, double *y, int64_t n);
 
 /* ---- diagnostics ---------------------------------------------------------- */
 

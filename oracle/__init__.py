@@ -53,6 +53,11 @@ def lib() -> C.CDLL:
         "vtl_ref_colsum_f64": (None, [vp, i64, i64, vp]),
         "vtl_ref_linear_backward_f32": (None, [vp, vp, vp, vp, vp, vp, i64, i64, i64, ci]),
         "vtl_ref_linear_backward_f64": (None, [vp, vp, vp, vp, vp, vp, i64, i64, i64, ci]),
+        "vtl_ref_gemv_f32": (None, [vp, vp, vp, i64, i64]),
+        "vtl_ref_gemv_f64": (None, [vp, vp, vp, i64, i64]),
+        "vtl_ref_sigmoid_f32": (None, [vp, vp, i64]),
+        "vtl_ref_sigmoid_f64": (None, [vp, vp, i64]),
+        "vtl_ref_relu_f64": (None, [vp, i64]),
         "vtl_ref_quantize_f32_i8_mt": (None, [vp, i64, i64, ci, vp, vp, ci]),
         "vtl_ref_dequantize_i8_f32_mt": (None, [vp, vp, i64, i64, ci, vp, ci]),
         "vtl_ref_max_threads": (ci, []),
@@ -240,3 +245,26 @@ def linear_backward(grad: np.ndarray, x: np.ndarray, w: np.ndarray, threads: int
     getattr(lib(), f"vtl_ref_linear_backward_{sfx}")(_p(grad), _p(x), _p(w), _p(dx), _p(dw), _p(db),
                                                      M, N, K, threads)
     return dx, dw, db
+
+
+def gemv(a: np.ndarray, x: np.ndarray) -> np.ndarray:
+    sfx = _suffix(a.dtype)
+    a, x = _c(a, a.dtype), _c(x, a.dtype)
+    assert a.ndim == 2 and x.shape == (a.shape[1],)
+    y = np.empty(a.shape[0], a.dtype)
+    getattr(lib(), f"vtl_ref_gemv_{sfx}")(_p(a), _p(x), _p(y), a.shape[0], a.shape[1])
+    return y
+
+
+def sigmoid(x: np.ndarray) -> np.ndarray:
+    sfx = _suffix(x.dtype)
+    x = _c(x, x.dtype)
+    y = np.empty_like(x)
+    getattr(lib(), f"vtl_ref_sigmoid_{sfx}")(_p(x), _p(y), x.size)
+    return y
+
+
+def relu_f64(x: np.ndarray) -> np.ndarray:
+    y = np.array(x, dtype=np.float64, copy=True, order="C")
+    lib().vtl_ref_relu_f64(_p(y), y.size)
+    return y

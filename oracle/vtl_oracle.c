@@ -38,6 +38,12 @@
  *                               benchmarks/vs_numpy/matmul_bench.v:28-33 in
  *                               closed form.  Same caveat on VSL's order.
  *   vtl_ref_colsum_f32/_f64     math.fsum (exact sum, one rounding).
+ *   vtl_ref_gemv_*              numpy f64 dot, integer-valued operands (exact).
+ *   vtl_ref_sigmoid_*           closed forms (sigmoid(0) = 0.5, sigmoid(x) +
+ *                               sigmoid(-x) = 1 to rounding), numpy's
+ *                               1 / (1 + exp(-x)) op by op; saturation at
+ *                               large |x|.  exp is the C library's, correct to
+ *                               <= 1 ulp: results pinned to that.
  *   vtl_ref_linear_backward_*   autograd_cuda/device_session_test.v:52-60
  *                               operands worked by hand (dx = [0.3, 0.45,
  *                               0.6], dw = [[1,2,3],[0.5,1,1.5]], db = grad),
@@ -279,6 +285,40 @@ VTL_REF_COLSUM(vtl_ref_colsum_f64, double)
     }
 VTL_REF_LINEAR_BACKWARD(vtl_ref_linear_backward_f32, float, vtl_ref_matmul_f32, vtl_ref_colsum_f32)
 VTL_REF_LINEAR_BACKWARD(vtl_ref_linear_backward_f64, double, vtl_ref_matmul_f64, vtl_ref_colsum_f64)
+
+#define VTL_REF_GEMV(NAME, T)                                                  \
+    void NAME(const T *A, const T *x, T *y, int64_t rows, int64_t cols)        \
+    {                                                                          \
+        for (int64_t r = 0; r < rows; r++) {                                   \
+            double acc = 0.0;                                                  \
+            for (int64_t c = 0; c < cols; c++)                                 \
+                acc += (double)A[r * cols + c] * (double)x[c];                 \
+            y[r] = (T)acc;                                                     \
+        }                                                                      \
+    }
+VTL_REF_GEMV(vtl_ref_gemv_f32, float)
+VTL_REF_GEMV(vtl_ref_gemv_f64, double)
+
+void vtl_ref_sigmoid_f32(const float *x, float *y, int64_t n)
+{
+    for (int64_t i = 0; i < n; i++) {
+        const float e = (float)exp(-(double)x[i]); /* vtl.cast[T](math.exp(-vtl.cast[f64](val))) */
+        y[i] = 1.0f / (1.0f + e);
+    }
+}
+
+void vtl_ref_sigmoid_f64(const double *x, double *y, int64_t n)
+{
+    for (int64_t i = 0; i < n; i++)
+        y[i] = 1.0 / (1.0 + exp(-x[i]));
+}
+
+void vtl_ref_relu_f64(double *x, int64_t n)
+{
+    for (int64_t i = 0; i < n; i++)
+        if (x[i] < 0.0)
+            x[i] = 0.0;
+}
 
 /* Row-parallel forms of the two bandwidth-bound routines, used only to time
  * the CPU baseline on all host cores.  Same arithmetic per element. */

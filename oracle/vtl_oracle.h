@@ -126,6 +126,19 @@ void vtl_ref_linear_backward_f32(const float *grad, const float *x, const float 
 void vtl_ref_linear_backward_f64(const double *grad, const double *x, const double *w, double *dx,
                                  double *dw, double *db, int64_t M, int64_t N, int64_t K, int threads);
 
+/* y[r] = sum_c A[r,c] * x[c] through f64, one rounding (gemv_cuda
+ * tensor_cuda_d_cuda.v:182-203; la.matmul arithmetic la/la.v:44-53). */
+void vtl_ref_gemv_f32(const float *A, const float *x, float *y, int64_t rows, int64_t cols);
+void vtl_ref_gemv_f64(const double *A, const double *x, double *y, int64_t rows, int64_t cols);
+
+/* y = 1 / (1 + T(exp(-f64(x)))), sum and quotient in T
+ * (nn/internal/activation.v:35-40). */
+void vtl_ref_sigmoid_f32(const float *x, float *y, int64_t n);
+void vtl_ref_sigmoid_f64(const double *x, double *y, int64_t n);
+
+/* ReLU on f64 in place (nn/internal/activation.v:63-70). */
+void vtl_ref_relu_f64(double *x, int64_t n);
+
 /* Row-parallel forms (same arithmetic), for timing the CPU baseline on all cores. */
 void vtl_ref_quantize_f32_i8_mt(const float *x, int64_t rows, int64_t cols, int per_row,
                                 int8_t *q, float *scale_out, int threads);

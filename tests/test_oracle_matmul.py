@@ -135,3 +135,44 @@ def test_empty_contraction_gives_zeros():
         c = oracle.matmul(np.zeros((3, 0), dt), np.zeros((0, 4), dt))
         assert c.shape == (3, 4) and not c.any()
         assert not oracle.colsum(np.zeros((0, 5), dt)).any()
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_gemv_against_numpy_and_exact_integers(dt):
+    rng = np.random.default_rng(15)
+    a, x = rng.standard_normal((37, 301)).astype(dt), rng.standard_normal(301).astype(dt)
+    got = oracle.gemv(a, x)
+    want = a.astype(np.float64) @ x.astype(np.float64)
+    if dt == np.float32:
+        assert ulp_diff(got, want.astype(np.float32)).max() <= 1
+    else:
+        assert np.all(np.abs(got - want) <= 1e-13 * (np.abs(a) @ np.abs(x)))
+    ai, xi = rng.integers(-9, 10, (50, 777)), rng.integers(-9, 10, 777)
+    assert np.array_equal(oracle.gemv(ai.astype(dt), xi.astype(dt)).astype(np.int64), ai @ xi)
+
+
+def test_sigmoid_closed_forms_and_numpy():
+    for dt in (np.float32, np.float64):
+        assert oracle.sigmoid(np.zeros(3, dt))[0] == dt(0.5)
+        x = np.linspace(-30, 30, 2001).astype(dt)
+        s = oracle.sigmoid(x)
+        assert s.dtype == dt and np.all((s >= 0) & (s <= 1)) and np.all(np.diff(s) >= 0)
+        # sigmoid(x) + sigmoid(-x) = 1 up to the roundings of the two quotients
+        assert np.all(np.abs(s + oracle.sigmoid(-x) - 1) <= 4 * np.finfo(dt).eps)
+        # the same three operations with numpy's exp (both exps are correct to <= 1 ulp of f64)
+        e = np.exp(-x.astype(np.float64)).astype(dt)
+        want = dt(1) / (dt(1) + e)
+        # one ulp of difference between the two exps can grow to two in the f64 quotient
+        assert ulp_diff(s, want.astype(dt)).max() <= (1 if dt == np.float32 else 2)
+        big = oracle.sigmoid(np.array([1000.0, -1000.0, 90.0, -90.0], dt))
+        assert big[0] == 1 and big[1] == 0 and big[2] == 1 and 0 <= big[3] < 1e-38
+    # literals: sigmoid(1) = 0.7310585786300049, sigmoid(-2) = 0.11920292202211755
+    s = oracle.sigmoid(np.array([1.0, -2.0]))
+    assert abs(s[0] - 0.7310585786300049) < 2e-16 and abs(s[1] - 0.11920292202211755) < 2e-17
+
+
+def test_relu_f64_closed_form():
+    x = np.array([-1.5, -0.0, 0.0, 2.5, -np.inf, np.inf, np.nan])
+    y = oracle.relu_f64(x)
+    assert np.array_equal(y[:6], [0.0, -0.0, 0.0, 2.5, 0.0, np.inf]) and np.isnan(y[6])
+    assert np.signbit(y[1]) and not np.signbit(y[0])

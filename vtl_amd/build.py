@@ -11,7 +11,7 @@ REPO_ROOT = os.path.dirname(PKG_DIR)
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libvtlhip.so")
 OBJ_DIR = os.path.join(PKG_DIR, "_build")
-SOURCES = ["runtime.hip", "quant.hip", "gemm_i8.hip", "matmul_f64acc.hip"]
+SOURCES = ["runtime.hip", "quant.hip", "gemm_i8.hip", "matmul_f64acc.hip", "tensor_ops.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

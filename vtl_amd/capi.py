@@ -57,6 +57,11 @@ SIGNATURES = {
     "vtl_hip_linear_backward_f32": (_ci, [_vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci]),
     "vtl_hip_linear_backward_f64": (_ci, [_vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci]),
     "vtl_hip_relu_f32": (_ci, [_vp, _i64]),
+    "vtl_hip_relu_f64": (_ci, [_vp, _i64]),
+    "vtl_hip_gemv_f32": (_ci, [_vp, _vp, _vp, _i64, _i64]),
+    "vtl_hip_gemv_f64": (_ci, [_vp, _vp, _vp, _i64, _i64]),
+    "vtl_hip_sigmoid_f32": (_ci, [_vp, _vp, _i64]),
+    "vtl_hip_sigmoid_f64": (_ci, [_vp, _vp, _i64]),
     "vtl_hip_strerror": (C.c_char_p, [_ci]),
     "vtl_hip_last_error": (C.c_char_p, []),
     "vtl_hip_version": (C.c_char_p, []),

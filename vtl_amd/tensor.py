@@ -136,9 +136,23 @@ class HipTensor:
 
     def relu_(self) -> "HipTensor":
         """In-place ReLU (x < 0 -> 0), cf. relu_cuda tensor_cuda_d_cuda.v:205-235."""
-        self._assert(np.float32, matrix=False, what="relu_")
-        capi.call("vtl_hip_relu_f32", self.ptr, self.size)
+        sfx = _float_suffix(self, "relu_")
+        capi.call(f"vtl_hip_relu_{sfx}", self.ptr, self.size)
         return self
+
+    def relu_hip(self) -> "HipTensor":
+        """`relu_hip() !&HipTensor[T]`: a new tensor, as relu_cuda (tensor_cuda_d_cuda.v:205-235)."""
+        out = HipTensor.empty(self.shape, self.dtype, HipParams(self.data.device_id))
+        capi.call("vtl_hip_memcpy_d2d", out.ptr, self.ptr, self.data.size)
+        return out.relu_()
+
+    def sigmoid_hip(self) -> "HipTensor":
+        """`sigmoid_hip() !&HipTensor[T]`: 1 / (1 + exp(-x)), as sigmoid_cuda
+        (tensor_cuda_d_cuda.v:237-270) with the arithmetic of nn/internal/activation.v:35-40."""
+        sfx = _float_suffix(self, "sigmoid_hip")
+        out = HipTensor.empty(self.shape, self.dtype, HipParams(self.data.device_id))
+        capi.call(f"vtl_hip_sigmoid_{sfx}", self.ptr, out.ptr, self.size)
+        return out
 
 
 def _per_row(axis: int) -> int:
@@ -286,3 +300,17 @@ def linear_backward_hip(grad: HipTensor, x: HipTensor, w: HipTensor, need_dx: bo
               dx.ptr if dx is not None else None, dw.ptr if dw is not None else None,
               db.ptr if db is not None else None, m, n, k)
     return [dx, dw, db]
+
+
+def gemv_hip(y: HipTensor, a: HipTensor, x: HipTensor) -> None:
+    """`gemv_hip(y, a, x) !`: y = A . x for A [m, n], x [n], y [m] (gemv_cuda,
+    tensor_cuda_d_cuda.v:182-203), f64 products and sums."""
+    sfx = _float_suffix(a, "gemv_hip")
+    if a.rank() != 2 or x.rank() != 1 or y.rank() != 1:
+        raise ValueError("gemv_hip: A must be rank-2, x and y must be rank-1")
+    if x.dtype != a.dtype or y.dtype != a.dtype:
+        raise TypeError("gemv_hip: operands of one type expected")
+    m, n = a.shape
+    if x.size != n or y.size != m:
+        raise ValueError(f"gemv_hip: A {a.shape}, x {x.shape}, y {y.shape}")
+    capi.call(f"vtl_hip_gemv_{sfx}", a.ptr, x.ptr, y.ptr, m, n)
