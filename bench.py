@@ -274,7 +274,7 @@ def bench_full_precision(timer: Timer, steps: int, warmup: int):
         "us": us, "TFLOP/s": tf,
         "roofline": {"bound": "mfma", "achieved": tf, "peak": PEAK_FP64_TFLOPS, "unit": "TFLOP/s",
                      "frac": tf / PEAK_FP64_TFLOPS, "traffic": None,
-                     "kernel": "matmul_f64acc_kernel<float, 128, 128, false, true, false, false>"}}
+                     "kernel": "matmul_f64acc_kernel<float, 2, 4, 4, 2, false, true, false, false>"}}
     for h in (X, W, B, Y):
         h.release()
 

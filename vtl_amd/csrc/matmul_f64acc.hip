@@ -75,11 +75,10 @@ __device__ __forceinline__ void read_operands(const T *__restrict__ p, double (&
 // One operand tile of BK x BMN elements (k-major in LDS, row stride LDW).
 // KMAJOR: the matrix is stored with the tile's m/n index contiguous ([K, MN]);
 // otherwise it is stored [MN, K] and is transposed on the way into LDS.
-template <typename T, int BK, int BMN, int LDW, bool KMAJOR, bool GUARD>
+template <typename T, int BK, int BMN, int LDW, int NT, bool KMAJOR, bool GUARD>
 struct OperandTile {
     static constexpr int kGroups = BK * BMN / 4;           // 4-element groups per tile
-    static constexpr int kPerThread = (kGroups + 255) / 256;
-    static_assert(kGroups % 256 == 0 || kGroups == 128, "tile must split over 256 threads");
+    static constexpr int kPerThread = (kGroups + NT - 1) / NT;   // NT threads in the workgroup
     Vec4<T> regs[kPerThread];
 
     // k_total: the matrix's K (its leading dimension when stored [MN, K]);
@@ -90,8 +89,8 @@ struct OperandTile {
         const int t = threadIdx.x;
 #pragma unroll
         for (int i = 0; i < kPerThread; ++i) {
-            const int g = t + 256 * i;
-            if (kGroups < 256 && g >= kGroups)
+            const int g = t + NT * i;
+            if (kGroups % NT != 0 && g >= kGroups)
                 break;
             if constexpr (KMAJOR) {
                 const int krow = g / (BMN / 4), c4 = g % (BMN / 4);
@@ -108,8 +107,8 @@ struct OperandTile {
         const int t = threadIdx.x;
 #pragma unroll
         for (int i = 0; i < kPerThread; ++i) {
-            const int g = t + 256 * i;
-            if (kGroups < 256 && g >= kGroups)
+            const int g = t + NT * i;
+            if (kGroups % NT != 0 && g >= kGroups)
                 break;
             if constexpr (KMAJOR) {
                 const int krow = g / (BMN / 4), c4 = g % (BMN / 4);
@@ -127,11 +126,13 @@ struct OperandTile {
 // GUARD == false: M, N, K are whole tiles and every row is 16-byte aligned, so
 // the loads and stores carry no bounds checks and the k-loop is straight-line code.
 // SPLIT: grid.y slices K; each slice writes its unrounded f64 sums to g.partial.
-template <typename T, int BM, int BN, bool TA, bool TB, bool GUARD, bool SPLIT>
-__global__ __launch_bounds__(256) void matmul_f64acc_kernel(const MatmulArgs g)
+// Workgroup = WR x WC waves, each with TM x TN MFMA tiles of 16x16:
+// BM = 16 * TM * WR, BN = 16 * TN * WC.
+template <typename T, int TM, int TN, int WR, int WC, bool TA, bool TB, bool GUARD, bool SPLIT>
+__global__ __launch_bounds__(64 * WR * WC) void matmul_f64acc_kernel(const MatmulArgs g)
 {
     constexpr int BK = 64 / (int)sizeof(T);   // 16 for f32, 8 for f64
-    constexpr int TM = BM / 32, TN = BN / 32; // MFMA tiles per wave in each direction
+    constexpr int BM = 16 * TM * WR, BN = 16 * TN * WC, NT = 64 * WR * WC;
     constexpr int LDA = BM + 4, LDB = BN + 4;
     static_assert(TM == 2 || TM == 4, "wave tile is 32 or 64 rows");
     static_assert(TN == 2 || TN == 4, "wave tile is 32 or 64 columns");
@@ -145,13 +146,13 @@ __global__ __launch_bounds__(256) void matmul_f64acc_kernel(const MatmulArgs g)
     const int m0 = (int)(blockIdx.x / tiles_n) * BM;
     const int n0 = (int)(blockIdx.x % tiles_n) * BN;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int wm = (wave >> 1) * (BM / 2), wn = (wave & 1) * (BN / 2);
+    const int wm = (wave / WC) * (16 * TM), wn = (wave % WC) * (16 * TN);
     const int r16 = lane & 15, kq = lane >> 4;
 
     // A as op(A)[M,K]: stored [K,M] when transposed (k-major already)
-    OperandTile<T, BK, BM, LDA, TA, GUARD> ta;
+    OperandTile<T, BK, BM, LDA, NT, TA, GUARD> ta;
     // B as op(B)[K,N]: stored [K,N] when not transposed (k-major already)
-    OperandTile<T, BK, BN, LDB, !TB, GUARD> tb;
+    OperandTile<T, BK, BN, LDB, NT, !TB, GUARD> tb;
 
     double4_t acc[TM][TN];
 #pragma unroll
@@ -363,32 +364,38 @@ __global__ __launch_bounds__(256) void matmul_splitk_finalize_kernel(const Matmu
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-template <typename T, int BM, int BN, bool GUARD, bool SPLIT>
+template <typename T, int TM, int TN, int WR, int WC, bool GUARD, bool SPLIT>
 int launch_tile_guard(const MatmulArgs &g, bool ta, bool tb, int splits, hipStream_t st)
 {
+    constexpr int BM = 16 * TM * WR, BN = 16 * TN * WC;
     const int64_t tiles = (int64_t)((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
     if (tiles > 0x7fffffff)
         return VTL_HIP_ERR_UNSUPPORTED;
-    const dim3 grid((unsigned)tiles, (unsigned)splits), block(256);
+    const dim3 grid((unsigned)tiles, (unsigned)splits), block(64 * WR * WC);
     if (!ta && !tb)
-        hipLaunchKernelGGL((matmul_f64acc_kernel<T, BM, BN, false, false, GUARD, SPLIT>), grid, block, 0, st, g);
+        hipLaunchKernelGGL((matmul_f64acc_kernel<T, TM, TN, WR, WC, false, false, GUARD, SPLIT>), grid, block, 0,
+                           st, g);
     else if (!ta && tb)
-        hipLaunchKernelGGL((matmul_f64acc_kernel<T, BM, BN, false, true, GUARD, SPLIT>), grid, block, 0, st, g);
+        hipLaunchKernelGGL((matmul_f64acc_kernel<T, TM, TN, WR, WC, false, true, GUARD, SPLIT>), grid, block, 0,
+                           st, g);
     else if (ta && !tb)
-        hipLaunchKernelGGL((matmul_f64acc_kernel<T, BM, BN, true, false, GUARD, SPLIT>), grid, block, 0, st, g);
+        hipLaunchKernelGGL((matmul_f64acc_kernel<T, TM, TN, WR, WC, true, false, GUARD, SPLIT>), grid, block, 0,
+                           st, g);
     else
-        hipLaunchKernelGGL((matmul_f64acc_kernel<T, BM, BN, true, true, GUARD, SPLIT>), grid, block, 0, st, g);
+        hipLaunchKernelGGL((matmul_f64acc_kernel<T, TM, TN, WR, WC, true, true, GUARD, SPLIT>), grid, block, 0,
+                           st, g);
     return check_launch("matmul_f64acc_kernel");
 }
 
 // Shapes made of whole tiles with 16-byte aligned rows run without bounds checks.
-template <typename T, int BM, int BN>
+template <typename T, int TM, int TN, int WR, int WC>
 int launch_tile(const MatmulArgs &g, bool ta, bool tb, hipStream_t st)
 {
+    constexpr int BM = 16 * TM * WR, BN = 16 * TN * WC;
     const bool whole = g.M % BM == 0 && g.N % BN == 0 && g.K % 16 == 0 && g.K > 0 && g.vec_a && g.vec_b &&
                        g.vec_c;
-    return whole ? launch_tile_guard<T, BM, BN, false, false>(g, ta, tb, 1, st)
-                 : launch_tile_guard<T, BM, BN, true, false>(g, ta, tb, 1, st);
+    return whole ? launch_tile_guard<T, TM, TN, WR, WC, false, false>(g, ta, tb, 1, st)
+                 : launch_tile_guard<T, TM, TN, WR, WC, true, false>(g, ta, tb, 1, st);
 }
 
 // Few output tiles and a long K: slice K over grid.y so that every SIMD holds
@@ -405,8 +412,8 @@ int launch_split(MatmulArgs g, bool ta, bool tb, int splits, hipStream_t st)
     if (!g.partial)
         return VTL_HIP_ERR_OUT_OF_MEMORY;
     const bool whole = g.M % 64 == 0 && g.N % 64 == 0 && g.K % per == 0 && g.vec_a && g.vec_b;
-    int rc = whole ? launch_tile_guard<T, 64, 64, false, true>(g, ta, tb, splits, st)
-                   : launch_tile_guard<T, 64, 64, true, true>(g, ta, tb, splits, st);
+    int rc = whole ? launch_tile_guard<T, 2, 2, 2, 2, false, true>(g, ta, tb, splits, st)
+                   : launch_tile_guard<T, 2, 2, 2, 2, true, true>(g, ta, tb, splits, st);
     if (rc != VTL_HIP_OK)
         return rc;
     const int64_t blocks = ((int64_t)g.M * g.N + 255) / 256;
@@ -442,8 +449,9 @@ int matmul_impl(const T *a, const T *b, T *c, const T *bias, int m, int n, int k
     hipStream_t st = current_stream();
     // 128x128 tiles once they fill the 256 compute units; 64x64 tiles otherwise
     const int64_t big = (int64_t)((m + 127) / 128) * ((n + 127) / 128);
+    // eight waves of 32x64 per 128x128 tile measured a few percent above four waves of 64x64
     if (big >= 192)
-        return launch_tile<T, 128, 128>(g, trans_a != 0, trans_b != 0, st);
+        return launch_tile<T, 2, 4, 4, 2>(g, trans_a != 0, trans_b != 0, st);
     const int64_t small = (int64_t)((m + 63) / 64) * ((n + 63) / 64);
     const char *force = getenv("VTL_HIP_MATMUL_SPLITS");   // tuning and tests
     int splits = force ? atoi(force) : 1;
@@ -456,7 +464,7 @@ int matmul_impl(const T *a, const T *b, T *c, const T *bias, int m, int n, int k
     }
     if (splits > 1 && k >= 32 * splits)
         return launch_split<T>(g, trans_a != 0, trans_b != 0, splits, st);
-    return launch_tile<T, 64, 64>(g, trans_a != 0, trans_b != 0, st);
+    return launch_tile<T, 2, 2, 2, 2>(g, trans_a != 0, trans_b != 0, st);
 }
 
 template <typename T>
