@@ -137,8 +137,13 @@ __global__ __launch_bounds__(64 * WR * WC) void matmul_f64acc_kernel(const Matmu
     static_assert(TM == 2 || TM == 4, "wave tile is 32 or 64 rows");
     static_assert(TN == 2 || TN == 4, "wave tile is 32 or 64 columns");
 
-    __shared__ __attribute__((aligned(16))) T As[2][BK * LDA];
-    __shared__ __attribute__((aligned(16))) T Bs[2][BK * LDB];
+    // Three LDS buffers per operand: while tile kt is multiplied, tile kt+1 is
+    // written at the start of the step (its global loads were issued a step
+    // earlier) and the one barrier per step sits before the last k-group, so
+    // that the first operands of tile kt+1 are read from LDS under the last
+    // MFMAs of tile kt and no MFMA waits for a barrier followed by an LDS read.
+    __shared__ __attribute__((aligned(16))) T As[3][BK * LDA];
+    __shared__ __attribute__((aligned(16))) T Bs[3][BK * LDB];
 
     const T *__restrict__ A = static_cast<const T *>(g.A);
     const T *__restrict__ B = static_cast<const T *>(g.B);
@@ -164,43 +169,60 @@ __global__ __launch_bounds__(64 * WR * WC) void matmul_f64acc_kernel(const Matmu
     const int k_begin = SPLIT ? (int)blockIdx.y * g.k_per_split : 0;
     const int k_end = SPLIT ? (k_begin + g.k_per_split < g.K ? k_begin + g.k_per_split : g.K) : g.K;
     const int ktiles = (k_end - k_begin + BK - 1) / BK;
+    constexpr int S = BK / 4;   // k-groups (one MFMA step each) per tile
+    const int aoff = wm + TM * r16 + kq * LDA, boff = wn + TN * r16 + kq * LDB;
+
     ta.fetch(A, g.M, g.K, k_end, m0, k_begin, g.vec_a != 0);
     tb.fetch(B, g.N, g.K, k_end, n0, k_begin, g.vec_b != 0);
     ta.stash(As[0]);
     tb.stash(Bs[0]);
+    if (ktiles > 1) {
+        ta.fetch(A, g.M, g.K, k_end, m0, k_begin + BK, g.vec_a != 0);
+        tb.fetch(B, g.N, g.K, k_end, n0, k_begin + BK, g.vec_b != 0);
+    }
     __syncthreads();
+    double a[TM], b[TN];
+    read_operands<T, TM>(As[0] + aoff, a);
+    read_operands<T, TN>(Bs[0] + boff, b);
 
+    int cur = 0;
     for (int kt = 0; kt < ktiles; ++kt) {
-        const int cur = kt & 1;
+        const int nxt = cur == 2 ? 0 : cur + 1;
         if (kt + 1 < ktiles) {
-            ta.fetch(A, g.M, g.K, k_end, m0, k_begin + (kt + 1) * BK, g.vec_a != 0);
-            tb.fetch(B, g.N, g.K, k_end, n0, k_begin + (kt + 1) * BK, g.vec_b != 0);
+            // buffer nxt was last read two steps ago; every wave has passed a barrier since
+            ta.stash(As[nxt]);
+            tb.stash(Bs[nxt]);
         }
-        const T *__restrict__ as = As[cur] + wm + TM * r16;
-        const T *__restrict__ bs = Bs[cur] + wn + TN * r16;
+        if (kt + 2 < ktiles) {
+            ta.fetch(A, g.M, g.K, k_end, m0, k_begin + (kt + 2) * BK, g.vec_a != 0);
+            tb.fetch(B, g.N, g.K, k_end, n0, k_begin + (kt + 2) * BK, g.vec_b != 0);
+        }
 #pragma unroll
-        for (int s = 0; s < BK / 4; ++s) {
-            const int k = 4 * s + kq;
-            double a[TM], b[TN];
-            read_operands<T, TM>(as + k * LDA, a);
-            read_operands<T, TN>(bs + k * LDB, b);
+        for (int s = 0; s < S; ++s) {
+            double an[TM], bn[TN];
+            if (s + 1 < S) {
+                read_operands<T, TM>(As[cur] + aoff + 4 * (s + 1) * LDA, an);
+                read_operands<T, TN>(Bs[cur] + boff + 4 * (s + 1) * LDB, bn);
+            } else {
+                __syncthreads();   // tile kt+1 is in LDS for every wave
+                read_operands<T, TM>(As[nxt] + aoff, an);
+                read_operands<T, TN>(Bs[nxt] + boff, bn);
+            }
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[i], b[j], acc[i][j], 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+                a[i] = an[i];
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                b[j] = bn[j];
         }
-        if (kt + 1 < ktiles) {
-            // the other buffer was last read before the barrier that ended the previous step
-            ta.stash(As[cur ^ 1]);
-            tb.stash(Bs[cur ^ 1]);
-        }
-        __syncthreads();
+        cur = nxt;
     }
 
-    // Element e of MFMA tile (i, j) in lane l is row 4 * e + l / 16, column
-    // l % 16 of that tile (the f64 16x16x4 layout): matrix row
-    // wm + TM * (4 * e + kq) + i, columns wn + TN * r16 + j (j contiguous).
     if constexpr (SPLIT) {
         double *__restrict__ P = g.partial + (int64_t)blockIdx.y * g.M * g.N;
         const int pcol0 = n0 + wn + TN * r16;
