@@ -5,7 +5,7 @@
 // Also the unquantized Linear forward (nn/layers/linear_forward_f32.v:16-18)
 // and LinearGate.backward (nn/gates/layers/linear.v:69-79) built on it.
 //
-// One workgroup of four waves owns a BM x BN tile of C.  Both operands are
+// One workgroup of WR x WC waves owns a BM x BN tile of C.  Both operands are
 // staged through LDS in k-major form (As[k][m], Bs[k][n]) whatever their
 // layout in memory, so that one 16- or 32-byte LDS read hands a lane the
 // operands of all its 16x16x4 MFMA tiles for one k.  MFMA tile i of a wave
