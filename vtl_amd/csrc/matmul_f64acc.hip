@@ -32,7 +32,7 @@ struct MatmulArgs {
     int M, N, K;
     int vec_a, vec_b, vec_c;   // base 16-byte aligned and leading dimension % 4 == 0
     int relu;
-    int k_per_split;           // split-K launches: k range of one grid.y slice (multiple of 16)
+    int k_per_split;           // split-K launches: k range of one grid.y slice (multiple of 32)
     double *partial;           // split-K launches: [splits][M][N] unrounded sums
 };
 
@@ -131,8 +131,9 @@ struct OperandTile {
 template <typename T, int TM, int TN, int WR, int WC, bool TA, bool TB, bool GUARD, bool SPLIT>
 __global__ __launch_bounds__(64 * WR * WC) void matmul_f64acc_kernel(const MatmulArgs g)
 {
-    constexpr int BK = 64 / (int)sizeof(T);   // 16 for f32, 8 for f64
     constexpr int BM = 16 * TM * WR, BN = 16 * TN * WC, NT = 64 * WR * WC;
+    // bytes of k per tile row: 64 (16 f32 / 8 f64); the small tile takes 128 to halve its barriers
+    constexpr int BK = (BM * BN <= 64 * 64 ? 128 : 64) / (int)sizeof(T);
     constexpr int LDA = BM + 4, LDB = BN + 4;
     static_assert(TM == 2 || TM == 4, "wave tile is 32 or 64 rows");
     static_assert(TN == 2 || TN == 4, "wave tile is 32 or 64 columns");
@@ -414,7 +415,7 @@ template <typename T, int TM, int TN, int WR, int WC>
 int launch_tile(const MatmulArgs &g, bool ta, bool tb, hipStream_t st)
 {
     constexpr int BM = 16 * TM * WR, BN = 16 * TN * WC;
-    const bool whole = g.M % BM == 0 && g.N % BN == 0 && g.K % 16 == 0 && g.K > 0 && g.vec_a && g.vec_b &&
+    const bool whole = g.M % BM == 0 && g.N % BN == 0 && g.K % 32 == 0 && g.K > 0 && g.vec_a && g.vec_b &&
                        g.vec_c;
     return whole ? launch_tile_guard<T, TM, TN, WR, WC, false, false>(g, ta, tb, 1, st)
                  : launch_tile_guard<T, TM, TN, WR, WC, true, false>(g, ta, tb, 1, st);
@@ -426,7 +427,7 @@ int launch_tile(const MatmulArgs &g, bool ta, bool tb, hipStream_t st)
 template <typename T>
 int launch_split(MatmulArgs g, bool ta, bool tb, int splits, hipStream_t st)
 {
-    const int per = ((g.K + splits - 1) / splits + 15) / 16 * 16;
+    const int per = ((g.K + splits - 1) / splits + 31) / 32 * 32;
     splits = (g.K + per - 1) / per;
     g.k_per_split = per;
     g.partial = static_cast<double *>(
@@ -469,12 +470,19 @@ int matmul_impl(const T *a, const T *b, T *c, const T *bias, int m, int n, int k
     g.k_per_split = 0;
     g.partial = nullptr;
     hipStream_t st = current_stream();
-    // 128x128 tiles once they fill the 256 compute units; 64x64 tiles otherwise
+    // Tile choice by a per-compute-unit estimate, in units of one 128x128 tile at
+    // peak: a compute unit runs two big workgroups together at ~0.84 of peak and
+    // a single one at ~0.75; the 64x64 tile kernel reaches 0.72 (four workgroups
+    // per compute unit) to 0.80 (nine and more) and quantizes four times finer
+    // over the 256 compute units.  Constants fitted to measured times.
     const int64_t big = (int64_t)((m + 127) / 128) * ((n + 127) / 128);
-    // eight waves of 32x64 per 128x128 tile measured a few percent above four waves of 64x64
-    if (big >= 192)
-        return launch_tile<T, 2, 4, 4, 2>(g, trans_a != 0, trans_b != 0, st);
     const int64_t small = (int64_t)((m + 63) / 64) * ((n + 63) / 64);
+    const int64_t c128 = (big + 255) / 256, c64 = (small + 255) / 256;
+    const double t128 = (double)(c128 / 2) * (2.0 / 0.84) + (double)(c128 % 2) * (1.0 / 0.75);
+    const double t64 = (double)c64 * 0.25 / (0.84 - 0.48 / (double)c64);
+    // eight waves of 32x64 per 128x128 tile measured a few percent above four waves of 64x64
+    if (t128 <= t64)
+        return launch_tile<T, 2, 4, 4, 2>(g, trans_a != 0, trans_b != 0, st);
     const char *force = getenv("VTL_HIP_MATMUL_SPLITS");   // tuning and tests
     int splits = force ? atoi(force) : 1;
     if (!force && small <= 512 && k >= 2048) {
