@@ -942,6 +942,21 @@ __global__ __launch_bounds__(256) void gemm_i8_small_kernel(const GemmArgs g)
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
+// A value per device: kernel attributes are per device, the library may serve several.
+template <typename V>
+struct PerDevice {
+    V v[64] = {};
+    V &get()
+    {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+            (void)hipGetLastError();
+            dev = 0;
+        }
+        return v[dev];
+    }
+};
+
 template <typename Kern>
 int launch_with_lds(Kern kern, bool &attr_done, int lds, int tiles, int threads, const GemmArgs &g,
                     hipStream_t st, const char *name)
@@ -974,21 +989,22 @@ int launch_dma(GemmArgs g, int splits, hipStream_t st)
         if (!g.partials)
             return VTL_HIP_ERR_OUT_OF_MEMORY;
     }
-    static bool done[4] = {false, false, false, false};
+    static PerDevice<bool> done_flags[4];
+    bool *done[4] = {&done_flags[0].get(), &done_flags[1].get(), &done_flags[2].get(), &done_flags[3].get()};
     const bool edge = (g.M % BM) || (g.N % BN);
     int rc;
     // the partial sums of a split launch are int32 whatever the final type is
     if (splits > 1 && edge)
-        rc = launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, false, true, true>, done[0], lds,
+        rc = launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, false, true, true>, *done[0], lds,
                              tiles * splits, 64 * WR * WC, g, st, "gemm_i8_dma_kernel");
     else if (splits > 1)
-        rc = launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, false, false, true>, done[1], lds,
+        rc = launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, false, false, true>, *done[1], lds,
                              tiles * splits, 64 * WR * WC, g, st, "gemm_i8_dma_kernel");
     else if (edge)
-        rc = launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, F32OUT, true, false>, done[2], lds,
+        rc = launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, F32OUT, true, false>, *done[2], lds,
                              tiles, 64 * WR * WC, g, st, "gemm_i8_dma_kernel");
     else
-        rc = launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, F32OUT, false, false>, done[3], lds,
+        rc = launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, F32OUT, false, false>, *done[3], lds,
                              tiles, 64 * WR * WC, g, st, "gemm_i8_dma_kernel");
     if (rc != VTL_HIP_OK || splits == 1)
         return rc;
@@ -1002,7 +1018,8 @@ int launch_tile(const GemmArgs &g, hipStream_t st)
 {
     constexpr int lds = 2 * (BM + BN) * 128;
     const int tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
-    static bool done = false;
+    static PerDevice<bool> done_flag;
+    bool &done = done_flag.get();
     return launch_with_lds(gemm_i8_tile_kernel<BM, BN, WR, WC, F32OUT>, done, lds, tiles, 64 * WR * WC, g, st,
                            "gemm_i8_tile_kernel");
 }
@@ -1070,7 +1087,8 @@ int launch_skinny_cfg(const GemmArgs &g, hipStream_t st)
 {
     constexpr int lds = NWAVE * STAGES * (8192 + XJ * 2048);
     static_assert(lds >= NWAVE * 4096, "room for the partial tiles");
-    static bool done = false;
+    static PerDevice<bool> done_flag;
+    bool &done = done_flag.get();
     const int blocks = (g.N + 31) / 32;
     return launch_with_lds(linear_skinny_kernel<NWAVE, STAGES, XJ, F32OUT>, done, lds, blocks, 64 * NWAVE, g, st,
                            "linear_skinny_kernel");
@@ -1094,7 +1112,8 @@ int launch_skinny_dynquant(const GemmArgs &g, hipStream_t st)
 {
     constexpr int NWAVE = 2, STAGES = 4;  // a deep ring: weights keep streaming while the rows are quantized
     const int lds = NWAVE * STAGES * 8192 + MR * (g.K + 16) + (MR + NWAVE * MR) * (int)sizeof(float) + 16;
-    static int attr_lds = 0;
+    static PerDevice<int> attr_lds_dev;
+    int &attr_lds = attr_lds_dev.get();
     auto kern = linear_skinny_dynquant_kernel<NWAVE, STAGES, MR>;
     if (lds > attr_lds) {  // the LDS need grows with K
         VTL_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
