@@ -8,7 +8,8 @@
 
 namespace vtlhip {
 
-static hipStream_t g_stream = nullptr;
+// per host thread, like HIP's current device: one host thread drives one device
+static thread_local hipStream_t g_stream = nullptr;
 static thread_local char g_last_error[256] = "";
 
 hipStream_t current_stream() { return g_stream; }
