@@ -68,7 +68,8 @@ int vtl_hip_memset(void *dst_device, int byte_value, size_t bytes);
 int vtl_hip_sync(void);
 
 /* Stream the compute entry points enqueue on (a hipStream_t, NULL = null
- * stream), kept per calling host thread like HIP's current device.  The reference has no stream concept beyond the unused field at
+ * stream), kept per calling host thread like HIP's current device.  The
+ * reference has no stream concept beyond the unused field at
  * storage/cuda_notd_cuda.v:9. */
 int vtl_hip_set_stream(void *hip_stream);
 int vtl_hip_get_stream(void **hip_stream);
