@@ -60,6 +60,28 @@ class Timer:
         capi.call("vtl_hip_event_elapsed_ms", self.e0, self.e1, C.byref(ms))
         return wall, float(ms.value)
 
+    def each(self, fn, steps: int):
+        """Median and minimum over `steps` launches timed one by one, in microseconds
+        (an event before every launch and one after the last; untimed by run())."""
+        steps = max(1, min(steps, 50))
+        evs = [C.c_void_p() for _ in range(steps + 1)]
+        for e in evs:
+            capi.call("vtl_hip_event_create", C.byref(e))
+        capi.call("vtl_hip_sync")
+        for i in range(steps):
+            capi.call("vtl_hip_event_record", evs[i])
+            fn()
+        capi.call("vtl_hip_event_record", evs[steps])
+        capi.call("vtl_hip_sync")
+        out = []
+        ms = C.c_float()
+        for i in range(steps):
+            capi.call("vtl_hip_event_elapsed_ms", evs[i], evs[i + 1], C.byref(ms))
+            out.append(float(ms.value) * 1e3)
+        for e in evs:
+            capi.call("vtl_hip_event_destroy", e)
+        return {"median_us": float(np.median(out)), "min_us": float(np.min(out))}
+
 
 def bench_linear(timer: Timer, steps: int, warmup: int, cpu: bool):
     m = n = k = 4096
@@ -76,7 +98,9 @@ def bench_linear(timer: Timer, steps: int, warmup: int, cpu: bool):
     wall, dev_ms = timer.run(step, steps)
     ops = 2.0 * m * n * k
     kernel_ms = dev_ms / steps
+    per_launch = timer.each(step, steps)
     res = {
+        "per_launch": per_launch,
         "ms_per_step": wall * 1e3 / steps,
         "tops": ops / (wall / steps) / 1e12,
         "roofline": {"kernel": "gemm_i8_dma_kernel<256,256,128,2,2,4,f32 epilogue>", "bound": "mfma",
@@ -131,9 +155,11 @@ def bench_quant(timer: Timer, steps: int, warmup: int, cpu: bool):
             fn()
         wall, dev_ms = timer.run(fn, steps)
         kernel_ms = dev_ms / steps
+        per_launch = timer.each(fn, steps)
         gbps = algo_bytes / (kernel_ms * 1e-3) / 1e9
         out[name] = {
             "value": algo_bytes / (wall / steps) / 1e9, "unit": "GB/s", "ms_per_step": wall * 1e3 / steps,
+            "per_launch": per_launch,
             "config": {"workload": f"configs[1]: per-row {name} of f32 [16384,16384], seed 1"},
             "roofline": {"kernel": kern, "bound": "hbm", "achieved": gbps, "peak": PEAK_HBM_GBPS,
                          "unit": "GB/s", "frac": gbps / PEAK_HBM_GBPS, "kernel_us": kernel_ms * 1e3,
@@ -239,8 +265,19 @@ def bench_other_configs(timer: Timer, steps: int, warmup: int):
     us = timed(c5)
     ops = 2.0 * m * sum(dims[i] * dims[i + 1] for i in range(3))
     wbytes = float(sum(dims[i] * dims[i + 1] for i in range(3)))
+    layers = {}
+    for i in range(3):
+        src = X if i == 0 else Ys[i - 1]
+
+        def one(i=i, src=src):
+            capi.call("vtl_hip_linear_f32_dynquant", src.ptr, Ws[i].ptr, Ss[i].ptr, None, Ys[i].ptr, m,
+                      dims[i + 1], dims[i], 1 if i < 2 else 0, ws.ptr, ws.size)
+        lus = timed(one)
+        layers[f"{dims[i]}->{dims[i + 1]}"] = {"us": lus, "TOPS": 2.0 * m * dims[i] * dims[i + 1] / lus / 1e6,
+                                               "weight_GB/s": dims[i] * dims[i + 1] / lus / 1e3}
     out["configs[4] int8 MLP chain 256x4096->11008->4096->1024"] = {
-        "us": us, "TOPS": ops / us / 1e6, "weight_GB/s": wbytes / us / 1e3, "ops": ops}
+        "us": us, "TOPS": ops / us / 1e6, "weight_GB/s": wbytes / us / 1e3, "ops": ops,
+        "per_layer (row quantize + int8 linear)": layers}
     capi.call("vtl_hip_sync")
     for h in Ws + Ss + Ys + [X]:
         h.release()
@@ -358,6 +395,7 @@ def main() -> int:
     }
     if lin:
         line["roofline"] = lin["roofline"]
+        line["per_launch"] = lin["per_launch"]
         if "cpu_baseline" in lin:
             line["cpu_baseline"] = lin["cpu_baseline"]
             line["cpu_baseline_all_cores"] = lin["cpu_baseline_all_cores"]
