@@ -180,3 +180,38 @@ def test_workload_generators_are_seeded_and_shaped():
     x, ws = workloads.mlp_chain(4, (64, 128, 32))
     assert x.shape == (4, 64) and [t.shape for t in ws] == [(128, 64), (32, 128)]
     assert np.abs(ws[0]).max() <= np.sqrt(6.0 / (64 + 128))
+
+
+def _header_arg_counts():
+    text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    out = {}
+    for name, args in re.findall(r"\b(vtl_hip_\w+)\s*\(([^)]*)\)\s*;", text):
+        args = args.strip()
+        out[name] = 0 if args in ("", "void") else len(args.split(","))
+    return out
+
+
+def test_v_binding_declarations_match_the_header():
+    """Every `fn C.vtl_hip_*` the V binding files declare exists in the header with the
+    same number of arguments, and the ctypes table agrees on the count too."""
+    counts = _header_arg_counts()
+    assert set(counts) == set(capi.SIGNATURES)
+    for name, (_, argtypes) in capi.SIGNATURES.items():
+        assert len(argtypes) == counts[name], name
+    vbind = os.path.join(ROOT, "vtl_amd", "vbind")
+    seen = set()
+    for dirpath, _, files in os.walk(vbind):
+        for f in files:
+            if not f.endswith(".v"):
+                continue
+            text = open(os.path.join(dirpath, f)).read()
+            for name, args in re.findall(r"fn C\.(vtl_hip_\w+)\(([^)]*)\)", text):
+                n = 0 if not args.strip() else len(args.split(","))
+                assert name in counts, f"{f}: {name} is not in vtl_hip.h"
+                assert n == counts[name], f"{f}: {name} takes {counts[name]} arguments, declared with {n}"
+                seen.add(name)
+    # the binding uses the compute surface of the library
+    for must in ("vtl_hip_quantize_f32_i8", "vtl_hip_dequantize_i8_f32", "vtl_hip_gemm_i8_i32", "vtl_hip_linear_i8_f32",
+                 "vtl_hip_linear_f32_dynquant", "vtl_hip_matmul_f32", "vtl_hip_linear_backward_f32",
+                 "vtl_hip_malloc", "vtl_hip_free", "vtl_hip_memcpy_h2d", "vtl_hip_memcpy_d2h"):
+        assert must in seen, must
