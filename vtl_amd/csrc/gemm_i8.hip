@@ -1031,7 +1031,7 @@ struct TileConfig {
     int wgs_per_cu;     // workgroups that fit a compute unit's LDS together
 };
 constexpr TileConfig kTileConfigs[] = {
-    {32, 64, 330.f, 1}, {32, 128, 520.f, 2}, {64, 128, 560.f, 2}, {128, 128, 830.f, 2}, {256, 256, 2600.f, 1}};
+    {32, 64, 330.f, 1}, {32, 128, 520.f, 2}, {64, 128, 640.f, 2}, {128, 128, 1150.f, 2}, {256, 256, 2600.f, 1}};
 constexpr int kNumTileConfigs = 5;
 
 template <bool F32OUT>
