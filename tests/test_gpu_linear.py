@@ -157,5 +157,16 @@ def test_single_token_fused_decode_equals_two_launch_path(hip, nk, monkeypatch):
     monkeypatch.delenv("VTL_HIP_NO_FUSED_DECODE")
     got = linear_f32_dynquant_hip(Z, W, SW, B, relu=False).cpu()
     assert np.array_equal(got, oracle.linear_f32_dynquant(np.zeros((1, k), np.float32), w, sw, bias))
+    # NaN elements are ignored by the absmax and quantize to 0; an infinite element makes the
+    # scale infinite and every code 0 -- the fused kernel follows the same rules
+    for special in (np.nan, np.inf, -np.inf):
+        xs = x.copy()
+        xs[0, 7] = special
+        xs[0, k - 1] = special
+        S = dev(xs)
+        got = linear_f32_dynquant_hip(S, W, SW, B, relu=False).cpu()
+        ref = oracle.linear_f32_dynquant(xs, w, sw, bias)
+        assert np.array_equal(got, ref, equal_nan=True), special
+        S.release()
     for h in (X, W, SW, B, Z):
         h.release()
