@@ -35,7 +35,7 @@ PEAK_FP64_TFLOPS = 78.6      # dense f64 MFMA, MI355X published
 # HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # script, each counter scaled by its reading for the 1 GiB copy_kernel (x2.000 and
 # x0.999); the summary of those runs is kept with the other profiler summaries.
-PMC_TRAFFIC_BYTES = {"linear": 168.1e6, "quantize": 1342.6e6, "dequantize": 1342.7e6}
+PMC_TRAFFIC_BYTES = {"linear": 168.1e6, "quantize": 1342.6e6, "dequantize": 1342.7e6, "linear_f32": 866.2e6}
 
 
 class Timer:
@@ -310,7 +310,7 @@ def bench_full_precision(timer: Timer, steps: int, warmup: int):
     out["linear_f32 (f64 accumulate) M=N=K=4096"] = {
         "us": us, "TFLOP/s": tf,
         "roofline": {"bound": "mfma", "achieved": tf, "peak": PEAK_FP64_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tf / PEAK_FP64_TFLOPS, "traffic": None,
+                     "frac": tf / PEAK_FP64_TFLOPS, "traffic": PMC_TRAFFIC_BYTES["linear_f32"],
                      "kernel": "matmul_f64acc_kernel<float, 2, 4, 4, 2, false, true, false, false>"}}
     for h in (X, W, B, Y):
         h.release()
