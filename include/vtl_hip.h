@@ -126,9 +126,11 @@ int vtl_hip_linear_i8_f32(const int8_t *A, const float *sa, int sa_per_row,
 
 /* Per-token (row) quantization of X[M,K] on the fly, then the int8 linear
  * against per-output-channel quantized weights.  workspace: device scratch
- * of at least vtl_hip_linear_f32_dynquant_workspace(M, K) bytes, owned by
- * the caller (the reference's DeviceSession keeps such staging buffers,
- * autograd_cuda/device_session.v:13-24). */
+ * of at least vtl_hip_linear_f32_dynquant_workspace(M, K) bytes, 16-byte
+ * aligned, owned by the caller (the reference's DeviceSession keeps such
+ * staging buffers, autograd_cuda/device_session.v:13-24); NULL (with size 0)
+ * makes the library stage in a buffer of its own, one per device, grown on
+ * demand. */
 size_t vtl_hip_linear_f32_dynquant_workspace(int M, int K);
 int vtl_hip_linear_f32_dynquant(const float *X, const int8_t *Wq, const float *sw,
                                 const float *bias, float *Y, int M, int N, int K, int relu,

@@ -67,7 +67,7 @@ def test_bad_arguments_return_status_not_abort():
     assert S("vtl_hip_gemm_i8_i32", one, one, one, -4, 4, 16) == E
     assert S("vtl_hip_gemm_i8_i32", one, one, one, 4, 4, 1 << 20) == capi.ERR_UNSUPPORTED
     assert S("vtl_hip_linear_i8_f32", one, None, 1, one, one, 1, None, one, 4, 4, 16, 0) == E
-    assert S("vtl_hip_linear_f32_dynquant", one, one, one, None, one, 4, 4, 16, 0, None, 0) == E
+    assert S("vtl_hip_linear_f32_dynquant", one, one, one, None, one, 4, 4, 16, 0, C.c_void_p(20), 4096) == E   # misaligned
     assert S("vtl_hip_linear_f32_dynquant", one, one, one, None, one, 4, 4, 16, 0, one, 8) == E
     assert S("vtl_hip_relu_f32", None, 4) == E
     assert S("vtl_hip_event_record", None) == E

@@ -170,3 +170,23 @@ def test_single_token_fused_decode_equals_two_launch_path(hip, nk, monkeypatch):
         S.release()
     for h in (X, W, SW, B, Z):
         h.release()
+
+
+@pytest.mark.parametrize("mnk", [(8, 2048, 4096), (256, 512, 11008), (37, 300, 1360), (1, 4096, 4096)])
+def test_dynquant_without_caller_workspace(hip, mnk):
+    """workspace = NULL: the library stages the quantized activations in a buffer of its
+    own, separate from the one its split-K launches use."""
+    m, n, k = mnk
+    rng = np.random.Generator(np.random.Philox(m + n + k))
+    x = rng.standard_normal((m, k), dtype=np.float32)
+    w = rng.integers(-127, 128, (n, k), dtype=np.int8)
+    sw = (rng.uniform(0.5, 1.5, n) * 1e-3).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    X, W, SW, B = dev(x), dev(w), dev(sw), dev(bias)
+    Y = HipTensor.empty([m, n], np.float32)
+    want = oracle.linear_f32_dynquant(x, w, sw, bias, relu=True, threads=CPU_THREADS)
+    for _ in range(2):
+        capi.call("vtl_hip_linear_f32_dynquant", X.ptr, W.ptr, SW.ptr, B.ptr, Y.ptr, m, n, k, 1, None, 0)
+        assert np.array_equal(Y.cpu(), want)
+    for h in (X, W, SW, B, Y):
+        h.release()

@@ -1221,14 +1221,14 @@ int vtl_hip_linear_f32_dynquant(const float *X, const int8_t *Wq, const float *s
     int st = check_gemm_args(X, Wq, Y, M, N, K);
     if (st != VTL_HIP_OK)
         return st;
-    if (!sw || !workspace)
+    if (!sw)
         return VTL_HIP_ERR_INVALID_ARG;
     if (M == 0 || N == 0)
         return VTL_HIP_OK;
     if (K == 0)
         return VTL_HIP_ERR_UNSUPPORTED;
-    if (workspace_bytes < vtl_hip_linear_f32_dynquant_workspace(M, K) ||
-        (reinterpret_cast<uintptr_t>(workspace) & 15))
+    if (workspace && (workspace_bytes < vtl_hip_linear_f32_dynquant_workspace(M, K) ||
+                      (reinterpret_cast<uintptr_t>(workspace) & 15)))
         return VTL_HIP_ERR_INVALID_ARG;
     if (M == 1 && K % 256 == 0 && K <= 4096 && N >= 2048 && aligned16(X) && aligned16(Wq) &&
         !getenv("VTL_HIP_NO_FUSED_DECODE")) {
@@ -1237,6 +1237,11 @@ int vtl_hip_linear_f32_dynquant(const float *X, const int8_t *Wq, const float *s
         // workspace stays unused.  VTL_HIP_NO_FUSED_DECODE forces the two-launch path (tests).
         GemmArgs g{nullptr, Wq, Y, nullptr, sw, bias, M, N, K, 1, 1, relu ? 1 : 0, 1, nullptr, X};
         return launch_skinny_dynquant<1>(g, current_stream());
+    }
+    if (!workspace) {   // no caller scratch: stage in the library's own buffer
+        workspace = vtlhip::library_workspace(vtl_hip_linear_f32_dynquant_workspace(M, K), 1);
+        if (!workspace)
+            return VTL_HIP_ERR_OUT_OF_MEMORY;
     }
     int8_t *xq = reinterpret_cast<int8_t *>(workspace);
     const size_t codes = (((size_t)M * (size_t)K) + 255) & ~(size_t)255;

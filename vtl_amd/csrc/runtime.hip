@@ -33,11 +33,15 @@ int check_launch(const char *kernel_name)
     return VTL_HIP_OK;
 }
 
-void *library_workspace(size_t bytes)
+void *library_workspace(size_t bytes, int slot)
 {
     constexpr int kMaxDevices = 64;
-    static void *buf[kMaxDevices] = {};
-    static size_t cap[kMaxDevices] = {};
+    static void *bufs[2][kMaxDevices] = {};
+    static size_t caps[2][kMaxDevices] = {};
+    if (slot < 0 || slot > 1)
+        return nullptr;
+    void **buf = bufs[slot];
+    size_t *cap = caps[slot];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
         (void)hipGetLastError();
