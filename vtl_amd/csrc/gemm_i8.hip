@@ -556,6 +556,16 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_skinny_kernel(const GemmArg
     }
 }
 
+// Workgroup barrier that orders LDS traffic only: unlike __syncthreads() it does
+// not wait for outstanding global loads, so direct-to-LDS weight loads issued
+// earlier stay in flight across it.
+__device__ __forceinline__ void lds_barrier()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
 // Decode with the activation quantization fused in, for M <= MR rows of f32
 // activations with K <= 4096 (used for a single token): every workgroup first computes the row scales itself
 // (absmax / 127 over the whole row - M x K floats from L2, cheap for a few rows)
@@ -605,27 +615,49 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_skinny_dynquant_kernel(cons
         for (int j = 0; j < LOADS; j++)
             __builtin_amdgcn_global_load_lds(VTL_GPTR(pw[j] + ko), VTL_LPTR(sw_ + j * 1024), 16, 0, 0);
     };
-    // weights first: they do not depend on the activations
-#pragma unroll
-    for (int st = 0; st < STAGES - 1; st++)
-        if (st < KC)
-            issue(st, st);
-
     // ---- row scales and codes of the activations: each row is read once and kept in
-    //      registers between the absmax pass and the quantize pass (K <= 4 * NT * RC) ----
+    //      registers between the absmax pass and the quantize pass (K <= 4 * NT * RC).
+    //      The activation loads are issued BEFORE the weight loads: vector-memory
+    //      results return in issue order, so the (cached) activations arrive first
+    //      and are quantized while the first weight chunks are still on their way ----
     constexpr int RC = 8;
     const int nv = K >> 2;
     float4_t xr[MR][RC];
     float mx[MR];
+    // The loads are written as instructions so that the wait below can name how
+    // many younger loads may stay in flight; the compiler's own bookkeeping would
+    // wait for the weight loads as well.  Lanes past the row re-read its last
+    // vector and discard it.
 #pragma unroll
     for (int m = 0; m < MR; m++) {
         const float4_t *xv = reinterpret_cast<const float4_t *>(g.xf32 + (int64_t)min(m, M - 1) * K);
 #pragma unroll
         for (int r = 0; r < RC; r++) {
             const int i = tid + r * NT;
-            xr[m][r] = (i < nv) ? xv[i] : float4_t{0.f, 0.f, 0.f, 0.f};
+            const float4_t *src = xv + (i < nv ? i : nv - 1);
+            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(xr[m][r]) : "v"(src) : "memory");
         }
     }
+    int issued = 0;
+#pragma unroll
+    for (int st = 0; st < STAGES - 1; st++)
+        if (st < KC) {
+            issue(st, st);
+            issued += LOADS;
+        }
+    // activations have arrived once at most the weight loads issued after them are outstanding
+    if (issued == (STAGES - 1) * LOADS)
+        wait_vmcnt<(STAGES - 1) * LOADS>();
+    else
+        wait_vmcnt<0>();
+#pragma unroll
+    for (int m = 0; m < MR; m++)
+#pragma unroll
+        for (int r = 0; r < RC; r++) {
+            asm volatile("" : "+v"(xr[m][r]));   // uses stay below the wait
+            if (tid + r * NT >= nv)
+                xr[m][r] = float4_t{0.f, 0.f, 0.f, 0.f};
+        }
 #pragma unroll
     for (int m = 0; m < MR; m++) {
         float a = 0.0f;
@@ -639,14 +671,14 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_skinny_dynquant_kernel(cons
         for (int m = 0; m < MR; m++)
             s_red[w * MR + m] = mx[m];
     }
-    __syncthreads();
+    lds_barrier();
     if (tid < MR) {
         float a = s_red[tid];
         for (int ww = 1; ww < NWAVE; ww++)
             a = fmaxf(a, s_red[ww * MR + tid]);
         s_scale[tid] = a / 127.0f;
     }
-    __syncthreads();
+    lds_barrier();
 #pragma unroll
     for (int m = 0; m < MR; m++) {
         const QuantScale p = make_quant_scale(s_scale[m]);
@@ -658,7 +690,7 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_skinny_dynquant_kernel(cons
                 dst[i] = quant4(xr[m][r], p);
         }
     }
-    __syncthreads();
+    lds_barrier();
 
     v16i acc0, acc1;
 #pragma unroll
