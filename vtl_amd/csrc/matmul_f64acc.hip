@@ -123,6 +123,16 @@ struct OperandTile {
     }
 };
 
+// Workgroup barrier that orders LDS traffic only: unlike __syncthreads() it does
+// not wait for outstanding global loads, so the operand loads issued two
+// k-tiles ahead stay in flight across it.
+__device__ __forceinline__ void lds_barrier()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
 // GUARD == false: M, N, K are whole tiles and every row is 16-byte aligned, so
 // the loads and stores carry no bounds checks and the k-loop is straight-line code.
 // SPLIT: grid.y slices K; each slice writes its unrounded f64 sums to g.partial.
@@ -205,7 +215,7 @@ __global__ __launch_bounds__(64 * WR * WC) void matmul_f64acc_kernel(const Matmu
                 read_operands<T, TM>(As[cur] + aoff + 4 * (s + 1) * LDA, an);
                 read_operands<T, TN>(Bs[cur] + boff + 4 * (s + 1) * LDB, bn);
             } else {
-                __syncthreads();   // tile kt+1 is in LDS for every wave
+                lds_barrier();   // tile kt+1 is in LDS for every wave; global loads stay in flight
                 read_operands<T, TM>(As[nxt] + aoff, an);
                 read_operands<T, TN>(Bs[nxt] + boff, bn);
             }
