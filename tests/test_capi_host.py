@@ -120,6 +120,11 @@ def test_predicates_and_matmul_shape_rule():
     assert a.is_matrix() and not a.is_vector() and not a.is_square_matrix()
     assert a.rank() == 2 and a.numel() == 64 and a.is_row_major() and not a.is_col_major()
     assert _fake([5, 5], np.float32).is_square_matrix() and _fake([5], np.float32).is_vector()
+    assert a.is_row_major_contiguous() and a.is_contiguous() and not a.is_col_major_contiguous()
+    t3 = _fake([2, 3, 4], np.float32)
+    assert t3.strides == [12, 4, 1] and t3.is_contiguous()
+    t3.strides = [12, 8, 1]                 # a strided view is not contiguous
+    assert not t3.is_row_major_contiguous() and not t3.is_contiguous()
     assert _matmul_shapes(a, w) == (4, 7, 16)
     with pytest.raises(ValueError, match="Invalid shapes for matrix multiplication"):   # la/la.v:41-43
         _matmul_shapes(a, _fake([7, 32], np.int8))

@@ -84,6 +84,24 @@ class HipTensor:
     def is_col_major(self) -> bool:
         return self.memory == "col_major"
 
+    def is_row_major_contiguous(self) -> bool:
+        """Strides are those of a dense row-major tensor (tensor_cuda_d_cuda.v:128-130)."""
+        return self.is_row_major() and self.strides == _strides_from_shape(self.shape)
+
+    def is_col_major_contiguous(self) -> bool:
+        """tensor_cuda_d_cuda.v:138-140; a device tensor is always uploaded row-major."""
+        if not self.is_col_major():
+            return False
+        strides, acc = [], 1
+        for d in self.shape:
+            strides.append(acc)
+            acc *= d
+        return self.strides == strides
+
+    def is_contiguous(self) -> bool:
+        """tensor_cuda_d_cuda.v:148-150."""
+        return self.is_row_major_contiguous() or self.is_col_major_contiguous()
+
     def _assert(self, dtype, matrix=True, what="tensor"):
         if self.dtype != np.dtype(dtype):
             raise TypeError(f"{what}: expected {np.dtype(dtype)}, got {self.dtype}")
