@@ -80,7 +80,8 @@ class Timer:
             out.append(float(ms.value) * 1e3)
         for e in evs:
             capi.call("vtl_hip_event_destroy", e)
-        return {"median_us": float(np.median(out)), "min_us": float(np.min(out))}
+        return {"median_us": float(np.median(out)), "min_us": float(np.min(out)),
+                "note": "launches separated by an event record each: includes that gap, unlike kernel_us"}
 
 
 def bench_linear(timer: Timer, steps: int, warmup: int, cpu: bool):
