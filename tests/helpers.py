@@ -1,5 +1,4 @@
 """Shared helpers of the GPU parity tests."""
-import ctypes as C
 import json
 import os
 from concurrent.futures import ThreadPoolExecutor

@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 
 from vtl_amd import capi, layers, workloads
-from vtl_amd.storage import HipParams, HipStorage
+from vtl_amd.storage import HipStorage
 from vtl_amd.tensor import HipTensor, _matmul_shapes, _per_row, _strides_from_shape
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))

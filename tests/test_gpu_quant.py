@@ -10,7 +10,6 @@ import pytest
 import oracle
 from helpers import KAT, d2h, dev, f32_list, h2d, quantize_with_scale_mt, raw_device_buffer, CPU_THREADS
 from vtl_amd import capi, workloads
-from vtl_amd.tensor import HipTensor
 
 pytestmark = pytest.mark.gpu
 

@@ -20,7 +20,7 @@ import json
 
 import numpy as np
 
-from .layers import PER_CHANNEL, PER_TENSOR, QuantLinearLayer
+from .layers import PER_CHANNEL, QuantLinearLayer
 
 MODEL_VERSION = "1.0"   # serialization.v:11
 
