@@ -103,7 +103,8 @@ int vtl_hip_device_info(char *name, size_t name_cap, int *compute_units, int *cl
     hipDeviceProp_t p;
     VTL_HIP_TRY(hipGetDeviceProperties(&p, dev));
     if (name && name_cap) {
-        snprintf(name, name_cap, "%s (%s)", p.name, p.gcnArchName);
+        // some driver stacks leave the marketing name empty
+        snprintf(name, name_cap, "%s (%s)", p.name[0] ? p.name : "AMD GPU", p.gcnArchName);
     }
     if (compute_units)
         *compute_units = p.multiProcessorCount;
