@@ -354,28 +354,56 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArg
 }
 
 // Sums the int32 partial results of a split-K launch (exact, order-free) and
-// applies the epilogue.  One thread per output element, n fastest.
-template <bool F32OUT>
+// applies the epilogue.  VEC consecutive outputs of one row per thread, n
+// fastest (VEC = 4 needs N % 4 == 0 and 16-byte aligned buffers).
+template <bool F32OUT, int VEC>
 __global__ __launch_bounds__(256) void splitk_finalize_kernel(const GemmArgs g)
 {
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) * VEC;
     const int64_t mn = (int64_t)g.M * g.N;
     if (idx >= mn)
         return;
-    int acc = 0;
-    for (int s = 0; s < g.splits; s++)
-        acc += g.partials[(int64_t)s * mn + idx];
+    int acc[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; j++)
+        acc[j] = 0;
+    for (int s = 0; s < g.splits; s++) {
+        const int32_t *p = g.partials + (int64_t)s * mn + idx;
+        if (VEC == 4) {
+            const v4i v = *reinterpret_cast<const v4i *>(p);
+#pragma unroll
+            for (int j = 0; j < VEC; j++)
+                acc[j] += v[j];
+        } else {
+            acc[0] += p[0];
+        }
+    }
     if (F32OUT) {
         const int m = (int)(idx / g.N), n = (int)(idx % g.N);
-        const float sc = g.sa[(int64_t)m * g.sa_stride] * g.sw[(int64_t)n * g.sw_stride];
-        float y = (float)acc * sc;
-        if (g.bias)
-            y = y + g.bias[n];
-        if (g.relu && y < 0.0f)
-            y = 0.0f;
-        reinterpret_cast<float *>(g.out)[idx] = y;
+        const float sa = g.sa[(int64_t)m * g.sa_stride];
+        float y[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; j++) {
+            const float sc = sa * g.sw[(int64_t)(n + j) * g.sw_stride];
+            y[j] = (float)acc[j] * sc;
+            if (g.bias)
+                y[j] = y[j] + g.bias[n + j];
+            if (g.relu && y[j] < 0.0f)
+                y[j] = 0.0f;
+        }
+        float *out = reinterpret_cast<float *>(g.out) + idx;
+        if (VEC == 4) {
+            *reinterpret_cast<vtlhip::qdev::float4_t *>(out) = vtlhip::qdev::float4_t{y[0], y[1], y[2], y[3]};
+        } else {
+            out[0] = y[0];
+        }
     } else {
-        reinterpret_cast<int32_t *>(g.out)[idx] = acc;
+        int32_t *out = reinterpret_cast<int32_t *>(g.out) + idx;
+        if (VEC == 4) {
+            *reinterpret_cast<v4i *>(out) = v4i{acc[0], acc[1], acc[2], acc[3]};
+        } else {
+            out[0] = acc[0];
+        }
     }
 }
 
@@ -1040,8 +1068,14 @@ int launch_dma(GemmArgs g, int splits, hipStream_t st)
                              tiles, 64 * WR * WC, g, st, "gemm_i8_dma_kernel");
     if (rc != VTL_HIP_OK || splits == 1)
         return rc;
-    const int64_t blocks = ((int64_t)g.M * g.N + 255) / 256;
-    hipLaunchKernelGGL((splitk_finalize_kernel<F32OUT>), dim3((unsigned)blocks), dim3(256), 0, st, g);
+    const int64_t mn = (int64_t)g.M * g.N;
+    if (g.N % 4 == 0 && aligned16(g.out) && aligned16(g.partials)) {
+        hipLaunchKernelGGL((splitk_finalize_kernel<F32OUT, 4>), dim3((unsigned)((mn / 4 + 255) / 256)), dim3(256), 0,
+                           st, g);
+    } else {
+        hipLaunchKernelGGL((splitk_finalize_kernel<F32OUT, 1>), dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, st,
+                           g);
+    }
     return check_launch("splitk_finalize_kernel");
 }
 
