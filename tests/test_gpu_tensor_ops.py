@@ -75,3 +75,17 @@ def test_sigmoid_and_relu(hip, dt):
     assert capi.status("vtl_hip_sigmoid_f32", None, None, 4) == capi.ERR_INVALID_ARG
     assert capi.status("vtl_hip_sigmoid_f64", None, None, 0) == capi.OK
     assert capi.status("vtl_hip_relu_f64", None, -1) == capi.ERR_INVALID_ARG
+
+
+def test_activation_hooks_host_round_trip(hip, monkeypatch):
+    from vtl_amd import relu_forward_hip_f32, sigmoid_forward_hip_f32
+    x = (np.random.default_rng(43).standard_normal((7, 33)) * 4).astype(np.float32)
+    monkeypatch.delenv("VTL_USE_HIP", raising=False)
+    with pytest.raises(RuntimeError, match="VTL_USE_HIP"):
+        relu_forward_hip_f32(x)
+    monkeypatch.setenv("VTL_USE_HIP", "1")
+    assert np.array_equal(relu_forward_hip_f32(x), oracle.relu(x))
+    assert ulp_diff(sigmoid_forward_hip_f32(x), oracle.sigmoid(x)).max() <= 1
+    assert relu_forward_hip_f32(np.zeros((0, 4), np.float32)).shape == (0, 4)
+    with pytest.raises(TypeError):
+        relu_forward_hip_f32(np.zeros(4, np.int32))

@@ -309,3 +309,42 @@ def linear_backward_hip_f32(grad: np.ndarray, input: np.ndarray, weight: np.ndar
         for t in (g_dev, x_dev, w_dev, *outs):
             if t is not None:
                 t.release()
+
+
+# -- activation hooks (cf. relu_forward_f32 / sigmoid_forward_f32,
+#    nn/layers/activation_forward_f32.v:7-24, and their Vulkan bodies
+#    nn/layers/activation_vulkan_d_vulkan.v:16-29) ---------------------------------
+
+def _activation_host_roundtrip(x, op: str) -> np.ndarray:
+    a = np.asarray(x)
+    if a.dtype not in (np.float32, np.float64):
+        raise TypeError(f"{op}: f32 or f64 tensor expected, got {a.dtype}")
+    if a.size == 0:
+        return a.copy()
+    t = HipTensor.from_host(a)
+    try:
+        if op == "relu":
+            return t.relu_().cpu()
+        out = t.sigmoid_hip()
+        try:
+            return out.cpu()
+        finally:
+            out.release()
+    finally:
+        t.release()
+
+
+def relu_forward_hip_f32(x: np.ndarray) -> np.ndarray:
+    """`relu_forward_hip_f32(x) !&vtl.Tensor[f32]`: ReLU through the device (x < 0 -> 0,
+    nn/internal/activation.v:63-70); the HIP body of relu_forward_f32's device branch."""
+    if not hip_linear_enabled():
+        raise RuntimeError("relu_forward_hip_f32: set VTL_USE_HIP=1 to enable")
+    return _activation_host_roundtrip(x, "relu")
+
+
+def sigmoid_forward_hip_f32(x: np.ndarray) -> np.ndarray:
+    """`sigmoid_forward_hip_f32(x) !&vtl.Tensor[f32]`: 1 / (1 + exp(-x)) through the device
+    with the arithmetic of nn/internal/activation.v:35-40."""
+    if not hip_linear_enabled():
+        raise RuntimeError("sigmoid_forward_hip_f32: set VTL_USE_HIP=1 to enable")
+    return _activation_host_roundtrip(x, "sigmoid")
