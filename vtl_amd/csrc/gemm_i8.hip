@@ -1138,7 +1138,7 @@ void choose_config(int M, int N, int K, int &best_idx, int &best_splits)
             const float throughput = (float)tiles * (float)s * (float)steps * c.step_cycles / 256.f + 3000.f;
             float cost = latency > throughput ? latency : throughput;
             if (s > 1)
-                cost += 6000.f + (float)s * (float)M * (float)N * 4.0f / 2500.f;
+                cost += 4500.f + (float)s * (float)M * (float)N * 4.0f / 2500.f;
             if (cost < best) {
                 best = cost;
                 best_idx = i;
