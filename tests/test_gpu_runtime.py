@@ -88,3 +88,34 @@ def test_unsupported_shapes_return_status(hip):
     assert capi.status("vtl_hip_linear_f32_dynquant", buf.ptr, buf.ptr, buf.ptr, None, buf.ptr, 8, 8, 64, 0,
                        buf.ptr + 4, 4000) == capi.ERR_INVALID_ARG
     buf.release()
+
+
+def test_compute_on_a_caller_stream(hip):
+    """vtl_hip_set_stream: the entry points enqueue on a stream the caller made (default
+    priority); results equal those on the null stream."""
+    import oracle
+    hiprt = C.CDLL("libamdhip64.so")
+    stream = C.c_void_p()
+    assert hiprt.hipStreamCreate(C.byref(stream)) == 0
+    try:
+        capi.call("vtl_hip_set_stream", stream)
+        got = C.c_void_p()
+        capi.call("vtl_hip_get_stream", C.byref(got))
+        assert got.value == stream.value
+        rng = np.random.default_rng(61)
+        x = rng.standard_normal((64, 1024)).astype(np.float32)
+        w = rng.integers(-127, 128, (256, 1024), dtype=np.int8)
+        sw = rng.uniform(0.5, 1.5, 256).astype(np.float32)
+        X, W, SW = HipTensor.from_host(x), HipTensor.from_host(w), HipTensor.from_host(sw)
+        Y = HipTensor.empty([64, 256], np.float32)
+        for _ in range(3):
+            capi.call("vtl_hip_linear_f32_dynquant", X.ptr, W.ptr, SW.ptr, None, Y.ptr, 64, 256, 1024, 1, None, 0)
+        capi.call("vtl_hip_sync")                      # waits on the caller's stream
+        assert np.array_equal(Y.cpu(), oracle.linear_f32_dynquant(x, w, sw, None, relu=True))
+        q, s = X.quantize_i8(0)
+        assert np.array_equal(q.dequantize(s, 0).cpu(), oracle.dequantize(*oracle.quantize(x, True), True))
+        for t in (X, W, SW, Y, q, s):
+            t.release()
+    finally:
+        capi.call("vtl_hip_set_stream", None)
+        assert hiprt.hipStreamDestroy(stream) == 0
