@@ -119,3 +119,51 @@ def test_compute_on_a_caller_stream(hip):
     finally:
         capi.call("vtl_hip_set_stream", None)
         assert hiprt.hipStreamDestroy(stream) == 0
+
+
+def test_entry_points_capture_into_a_hip_graph(hip):
+    """Quantize + int8 linear recorded once into a HIP graph on a caller stream and
+    replayed with new activations: every replay equals the oracle.  (The recorded
+    entry points allocate nothing and record no memset; kernel attributes are set
+    by a warm-up call before the capture.)"""
+    import oracle
+    hiprt = C.CDLL("libamdhip64.so")
+    stream, graph, gexec = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    assert hiprt.hipStreamCreate(C.byref(stream)) == 0
+    rng = np.random.default_rng(62)
+    m, n, k = 48, 512, 1024
+    w = rng.integers(-127, 128, (n, k), dtype=np.int8)
+    sw = rng.uniform(0.5, 1.5, n).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    X, W, SW, B = (HipTensor.from_host(a) for a in (x, w, sw, bias))
+    XQ, SX, Y = HipTensor.empty([m, k], np.int8), HipTensor.empty([m], np.float32), HipTensor.empty([m, n], np.float32)
+
+    def enqueue():
+        capi.call("vtl_hip_quantize_f32_i8", X.ptr, m, k, 1, XQ.ptr, SX.ptr)
+        capi.call("vtl_hip_linear_i8_f32", XQ.ptr, SX.ptr, 1, W.ptr, SW.ptr, 1, B.ptr, Y.ptr, m, n, k, 1)
+
+    try:
+        capi.call("vtl_hip_set_stream", stream)
+        enqueue()                                   # warm-up outside the capture
+        capi.call("vtl_hip_sync")
+        assert hiprt.hipStreamBeginCapture(stream, 0) == 0
+        enqueue()
+        assert hiprt.hipStreamEndCapture(stream, C.byref(graph)) == 0
+        assert hiprt.hipGraphInstantiate(C.byref(gexec), graph, None, None, C.c_size_t(0)) == 0
+        for rep in range(4):
+            xr = (rng.standard_normal((m, k)) * (rep + 1)).astype(np.float32)
+            capi.call("vtl_hip_memcpy_h2d", X.ptr, xr.ctypes.data, xr.nbytes)     # eager work between replays
+            assert hiprt.hipGraphLaunch(gexec, stream) == 0
+            capi.call("vtl_hip_sync")
+            wq_ref = oracle.linear_f32_dynquant(xr, w, sw, bias, relu=True)
+            assert np.array_equal(Y.cpu(), wq_ref), f"replay {rep}"
+    finally:
+        capi.call("vtl_hip_set_stream", None)
+        if gexec:
+            hiprt.hipGraphExecDestroy(gexec)
+        if graph:
+            hiprt.hipGraphDestroy(graph)
+        hiprt.hipStreamDestroy(stream)
+        for t in (X, W, SW, B, XQ, SX, Y):
+            t.release()
