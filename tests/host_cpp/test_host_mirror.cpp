@@ -2,6 +2,7 @@
 // oracle on a real device: alloc -> H2D -> op -> D2H -> release, plus the error
 // paths.  Links libvtlhip.so (product) and libvtloracle.so (checker).
 // Exit code 0 = all checks passed.
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -148,6 +149,41 @@ int main(int argc, char **argv)
         CHECK(got[0] == dx && got[1] == dw && got[2] == db);
         auto no_bias = vtl::linear_backward_hip_f32(g, M, N, xi, K, wi, false);
         CHECK(no_bias[0] == dx && no_bias[2] == std::vector<float>(N, 0.0f));
+    }
+    // generic tensor operations vs oracle
+    {
+        std::uniform_int_distribution<int> ud(-8, 8);
+        std::vector<double> a((size_t)M * K), xv(K), yr(M);
+        for (auto &v : a) v = ud(rng);
+        for (auto &v : xv) v = ud(rng);
+        auto A = vtl::HipTensor<double>::from_host(a, {M, K});
+        auto X = vtl::HipTensor<double>::from_host(xv, {K});
+        vtl::HipTensor<double> Y({M});
+        vtl::gemv_hip(Y, A, X);
+        vtl_ref_gemv_f64(a.data(), xv.data(), yr.data(), M, K);
+        CHECK(Y.cpu() == yr);                       // integer-valued: exact in any order
+        try {
+            vtl::gemv_hip(Y, A, Y);
+            CHECK(false);
+        } catch (const std::invalid_argument &) {
+        }
+        auto R = vtl::HipTensor<float>::from_host(x, {M, K});
+        vtl::relu_hip(R);
+        std::vector<float> rr = x;
+        vtl_ref_relu_f32(rr.data(), (int64_t)rr.size());
+        CHECK(R.cpu() == rr);
+        auto S = vtl::sigmoid_hip(xt);
+        std::vector<float> sr(x.size());
+        vtl_ref_sigmoid_f32(x.data(), sr.data(), (int64_t)x.size());
+        auto sg = S.cpu();
+        int worst = 0;
+        for (size_t i = 0; i < sr.size(); i++) {
+            int32_t u, v;
+            std::memcpy(&u, &sg[i], 4);
+            std::memcpy(&v, &sr[i], 4);
+            worst = std::max(worst, std::abs(u - v));
+        }
+        CHECK(worst <= 1);                          // the device's f64 exp against the C library's
     }
     std::printf(failures ? "host mirror: %d failure(s)\n" : "host mirror: ok\n", failures);
     return failures ? 1 : 0;

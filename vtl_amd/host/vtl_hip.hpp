@@ -258,6 +258,51 @@ inline HipTensor<T> matmul_hip(const HipTensor<T> &a, const HipTensor<T> &b, boo
     return c;
 }
 
+// `gemv_hip(y, a, x) !` (cf. gemv_cuda, tensor_cuda_d_cuda.v:182-203): y = A . x.
+template <typename T>
+inline void gemv_hip(HipTensor<T> &y, const HipTensor<T> &a, const HipTensor<T> &x)
+{
+    static_assert(std::is_same<T, float>::value || std::is_same<T, double>::value, "f32 or f64");
+    if (a.rank() != 2 || x.rank() != 1 || y.rank() != 1)
+        throw std::invalid_argument("gemv_hip: A must be rank-2, x and y must be rank-1");
+    if (x.size != (size_t)a.shape[1] || y.size != (size_t)a.shape[0])
+        throw std::invalid_argument("gemv_hip: shapes of A, x and y disagree");
+    if (std::is_same<T, float>::value)
+        hip_check(vtl_hip_gemv_f32((const float *)a.data.ptr, (const float *)x.data.ptr, (float *)y.data.ptr,
+                                   a.shape[0], a.shape[1]),
+                  "vtl_hip_gemv_f32");
+    else
+        hip_check(vtl_hip_gemv_f64((const double *)a.data.ptr, (const double *)x.data.ptr, (double *)y.data.ptr,
+                                   a.shape[0], a.shape[1]),
+                  "vtl_hip_gemv_f64");
+}
+
+// `sigmoid_hip() !&HipTensor[T]` (cf. sigmoid_cuda, tensor_cuda_d_cuda.v:237-270): a new tensor.
+template <typename T>
+inline HipTensor<T> sigmoid_hip(const HipTensor<T> &t)
+{
+    static_assert(std::is_same<T, float>::value || std::is_same<T, double>::value, "f32 or f64");
+    HipTensor<T> out(t.shape, HipParams{t.data.device_id});
+    if (std::is_same<T, float>::value)
+        hip_check(vtl_hip_sigmoid_f32((const float *)t.data.ptr, (float *)out.data.ptr, (int64_t)t.size),
+                  "vtl_hip_sigmoid_f32");
+    else
+        hip_check(vtl_hip_sigmoid_f64((const double *)t.data.ptr, (double *)out.data.ptr, (int64_t)t.size),
+                  "vtl_hip_sigmoid_f64");
+    return out;
+}
+
+// `relu_hip() !` in place (cf. relu_cuda, tensor_cuda_d_cuda.v:205-235).
+template <typename T>
+inline void relu_hip(HipTensor<T> &t)
+{
+    static_assert(std::is_same<T, float>::value || std::is_same<T, double>::value, "f32 or f64");
+    if (std::is_same<T, float>::value)
+        hip_check(vtl_hip_relu_f32((float *)t.data.ptr, (int64_t)t.size), "vtl_hip_relu_f32");
+    else
+        hip_check(vtl_hip_relu_f64((double *)t.data.ptr, (int64_t)t.size), "vtl_hip_relu_f64");
+}
+
 // `linear_backward_hip_f32(grad, input, weight, bias_needs_grad) ![]&vtl.Tensor[f32]`
 // (cf. linear_backward_vulkan_f32, nn/internal/linear_vulkan_backward_d_vulkan.v:9-38):
 // host tensors in, {d_input[M,K], d_weight[N,K], d_bias[1,N]} out; d_bias is zeros
