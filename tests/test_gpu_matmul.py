@@ -14,7 +14,8 @@ import pytest
 import oracle
 from helpers import CPU_THREADS, dev
 from vtl_amd import capi
-from vtl_amd.layers import linear_backward_hip_f32, linear_forward_hip_exact, matmul_hip_host
+from vtl_amd.layers import (linear_backward_hip_f32, linear_forward_hip_exact, matmul_gate_backward_hip,
+                            matmul_hip_host)
 from vtl_amd.tensor import colsum_hip, linear_backward_hip, linear_hip, matmul_hip
 
 pytestmark = pytest.mark.gpu
@@ -272,3 +273,23 @@ def test_argument_errors(hip):
     from helpers import d2h
     assert not d2h(p, 12, np.float32).any()
     buf.release()
+
+
+def test_matmul_gate_backward(hip, monkeypatch):
+    """MatMulGate.backward (autograd/gates_blas.v:43-48): dA = g . B^T, dB = A^T . g."""
+    monkeypatch.setenv("VTL_USE_HIP", "1")
+    monkeypatch.setenv("VTL_HIP_BACKWARD", "1")
+    rng = np.random.default_rng(28)
+    for dt in (np.float32, np.float64):
+        a = rng.standard_normal((37, 53)).astype(dt)
+        b = rng.standard_normal((53, 29)).astype(dt)
+        g = rng.standard_normal((37, 29)).astype(dt)
+        da, db = matmul_gate_backward_hip(g, a, b)
+        want_a = oracle.matmul(g, np.ascontiguousarray(b.T))
+        want_b = oracle.matmul(np.ascontiguousarray(a.T), g)
+        absa = np.abs(g).astype(np.float64) @ np.abs(b.T).astype(np.float64)
+        absb = np.abs(a.T).astype(np.float64) @ np.abs(g).astype(np.float64)
+        assert_close_to_oracle(da, want_a, absa)
+        assert_close_to_oracle(db, want_b, absb)
+    with pytest.raises(ValueError, match="Invalid shapes"):
+        matmul_gate_backward_hip(np.zeros((3, 3)), np.zeros((3, 4)), np.zeros((5, 3)))

@@ -9,7 +9,8 @@ from .layers import (PER_CHANNEL, PER_TENSOR, HipSession, QuantLinearLayer,  # n
                      QuantizedWeights, hip_backward_enabled, hip_linear_enabled,
                      hip_tests_enabled, linear_backward_hip_f32, linear_forward_f32_use_hip,
                      linear_forward_hip_exact, linear_forward_hip_f32,
-                     linear_gate_use_hip_backward, matmul_hip_host, relu_forward_hip_f32,
+                     linear_gate_use_hip_backward, matmul_gate_backward_hip, matmul_hip_host,
+                     relu_forward_hip_f32,
                      sigmoid_forward_hip_f32)
 from .models import Sequential  # noqa: F401
 from .storage import HipParams, HipStorage, hip_available  # noqa: F401

@@ -348,3 +348,24 @@ def sigmoid_forward_hip_f32(x: np.ndarray) -> np.ndarray:
     if not hip_linear_enabled():
         raise RuntimeError("sigmoid_forward_hip_f32: set VTL_USE_HIP=1 to enable")
     return _activation_host_roundtrip(x, "sigmoid")
+
+
+def matmul_gate_backward_hip(grad: np.ndarray, a: np.ndarray, b: np.ndarray):
+    """`MatMulGate.backward` (autograd/gates_blas.v:43-48) through the device:
+    [grad . b^T, a^T . grad], the transposes taken by flag instead of `.t()` copies."""
+    if not hip_backward_enabled():
+        raise RuntimeError("matmul_gate_backward_hip: set VTL_USE_HIP=1 and VTL_HIP_BACKWARD=1")
+    g = _as_float_matrix(grad, "matmul backward")
+    av = _as_float_matrix(a, "matmul backward").astype(g.dtype, copy=False)
+    bv = _as_float_matrix(b, "matmul backward").astype(g.dtype, copy=False)
+    if av.shape[1] != bv.shape[0] or g.shape != (av.shape[0], bv.shape[1]):
+        raise ValueError(f"Invalid shapes for matrix multiplication {list(av.shape)} and {list(bv.shape)}")
+    g_dev, a_dev, b_dev = HipTensor.from_host(g), HipTensor.from_host(av), HipTensor.from_host(bv)
+    outs = []
+    try:
+        outs.append(matmul_hip(g_dev, b_dev, False, True))    # [M,N] . [K,N]^T -> [M,K]
+        outs.append(matmul_hip(a_dev, g_dev, True, False))    # [M,K]^T . [M,N] -> [K,N]
+        return [t.cpu() for t in outs]
+    finally:
+        for t in (g_dev, a_dev, b_dev, *outs):
+            t.release()
