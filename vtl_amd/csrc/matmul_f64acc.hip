@@ -15,8 +15,6 @@
 
 #include <stdlib.h>
 
-#include <type_traits>
-
 namespace {
 
 using vtlhip::check_launch;
