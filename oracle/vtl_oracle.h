@@ -105,8 +105,12 @@ void vtl_ref_linear_f32_via_f64(const float *X, const float *W, const float *bia
  * [M,K] row-major, else A is stored [K,M] (the caller's `.t()`, as in
  * MatMulGate.backward gates_blas.v:43-48 and LinearGate.backward
  * nn/gates/layers/linear.v:69-74); same for B ([K,N] / [N,K]).  threads > 1:
- * OpenMP over rows, same arithmetic.  Summation order inside VSL's GEMM is
- * unknown: parity unpinned beyond f64 rounding error. */
+ * OpenMP over rows, same arithmetic.  Summation order inside VSL's GEMM
+ * (vsl@v0.2.0-beta.1, not vendored) is unknown and is not even one order: the
+ * reference's CI builds it both over its pure-V BLAS and over cblas
+ * (.github/workflows/ci.yml:81-86,132-140), so the reference's own f32 results
+ * are defined only up to the order of the f64 sum.  Parity unpinned beyond
+ * that f64 rounding error (about 1e-16 relative before the one rounding). */
 void vtl_ref_matmul_f32(const float *A, const float *B, float *C, int64_t M, int64_t N, int64_t K,
                         int trans_a, int trans_b, int threads);
 void vtl_ref_matmul_f64(const double *A, const double *B, double *C, int64_t M, int64_t N, int64_t K,
