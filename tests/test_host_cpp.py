@@ -30,3 +30,14 @@ def test_host_mirror_on_device(hip):
     res = subprocess.run([BIN], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
     assert res.returncode == 0, res.stdout
     assert "host mirror: ok" in res.stdout
+
+
+def test_plain_c_consumer_of_the_abi():
+    """tests/host_c/abi_check.c is C99 -pedantic -Werror: the header is valid C, the
+    exports have C linkage, argument checks answer without a device."""
+    cdir = os.path.join(HERE, "host_c")
+    exe = os.path.join(cdir, "abi_check")
+    if not os.path.exists(exe):   # built by __graft_entry__.build(); this is the CPU-side fallback
+        subprocess.run(["make", "-C", cdir], check=True, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
+    res = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=60)
+    assert res.returncode == 0 and "C ABI check: ok" in res.stdout, res.stdout
