@@ -1299,7 +1299,8 @@ int vtl_hip_linear_f32_dynquant(const float *X, const int8_t *Wq, const float *s
     if (M == 1 && K % 256 == 0 && K <= 4096 && N >= 2048 && aligned16(X) && aligned16(Wq) &&
         !getenv("VTL_HIP_NO_FUSED_DECODE")) {
         // a single token: quantize it inside the weight-streaming kernel (one launch instead of
-        // two; measured 9 % faster at N = 14336, K = 4096, and slower from two rows on).  The
+        // two; measured 15 % faster at N = 14336, K = 4096; for two rows 13.5 us against 12.8 us
+        // for the two launches, and from three rows on the registers no longer hold the rows).  The
         // workspace stays unused.  VTL_HIP_NO_FUSED_DECODE forces the two-launch path (tests).
         GemmArgs g{nullptr, Wq, Y, nullptr, sw, bias, M, N, K, 1, 1, relu ? 1 : 0, 1, nullptr, X};
         return launch_skinny_dynquant<1>(g, current_stream());
