@@ -226,8 +226,9 @@ def bench_other_configs(timer: Timer, steps: int, warmup: int):
     # configs[3]: K=4096, N=14336, M in {1,8,32,128}
     k, n = 4096, 14336
     rng = np.random.Generator(np.random.Philox(3))
-    Wq = HipTensor.from_host(rng.integers(-127, 128, (n, k), dtype=np.int8))
-    Sw = HipTensor.from_host((rng.uniform(0.5, 1.5, n) * 1e-3).astype(np.float32))
+    W = HipTensor.from_host(rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02))
+    Wq, Sw = W.quantize_i8(0)                      # one scale per output channel
+    W.release()
     dec = {}
     for m in (1, 8, 32, 128):
         X = HipTensor.from_host(rng.standard_normal((m, k), dtype=np.float32))
@@ -251,8 +252,14 @@ def bench_other_configs(timer: Timer, steps: int, warmup: int):
 
     # configs[4]: 256x4096 -> 11008 -> ReLU -> 4096 -> ReLU -> 1024, device-resident chain
     dims, m = (4096, 11008, 4096, 1024), 256
-    Ws = [HipTensor.from_host(rng.integers(-127, 128, (dims[i + 1], dims[i]), dtype=np.int8)) for i in range(3)]
-    Ss = [HipTensor.from_host((rng.uniform(0.5, 1.5, dims[i + 1]) * 1e-3).astype(np.float32)) for i in range(3)]
+    Ws, Ss = [], []
+    for i in range(3):                             # Xavier-uniform f32 weights, one scale per output channel
+        bound = np.float32(np.sqrt(6.0 / (dims[i] + dims[i + 1])))
+        W = HipTensor.from_host((rng.random((dims[i + 1], dims[i]), dtype=np.float32) * 2 - 1) * bound)
+        wq, sw = W.quantize_i8(0)
+        W.release()
+        Ws.append(wq)
+        Ss.append(sw)
     X = HipTensor.from_host(rng.standard_normal((m, dims[0]), dtype=np.float32))
     Ys = [HipTensor.empty([m, dims[i + 1]], np.float32) for i in range(3)]
     ws = HipStorage.empty(int(capi.lib().vtl_hip_linear_f32_dynquant_workspace(m, max(dims))), np.uint8)
