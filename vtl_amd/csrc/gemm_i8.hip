@@ -287,6 +287,36 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArg
             for (int j = 0; j < TN; j++)
                 acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[buf][i], bf[buf][j], acc[i][j], 0, 0, 0);
     };
+    // The last k-step of a tile with the next tile's loads issued between its
+    // MFMAs, a few after each, in a fixed order.  Issued in one burst right
+    // after the barrier, the loads of all waves pile up in front of the compute
+    // unit's one address unit and the in-order waves stall behind them instead
+    // of issuing MFMAs.
+    auto mma_issue = [&](int buf, int kt, int st) {
+        constexpr int NM = TM * TN, PER = (LPT + NM - 1) / NM;  // loads after each MFMA
+        char *sa_ = smem + st * STAGE;
+        char *sb_ = sa_ + BM * BK;
+        const int64_t ko = (int64_t)(kt_begin + kt) * BK;
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int q = 0; q < NM; q++) {
+            acc[q / TN][q % TN] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[buf][q / TN], bf[buf][q % TN],
+                                                                        acc[q / TN][q % TN], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int d = q * PER; d < (q + 1) * PER && d < LPT; d++) {
+                if (d < A_PW)
+                    __builtin_amdgcn_global_load_lds(
+                        VTL_GPTR(EDGE ? pa[EDGE ? d : 0] + ko : pa[0] + ko + d * jstride),
+                        VTL_LPTR(sa_ + (w + NW * d) * 1024), 16, 0, 0);
+                else
+                    __builtin_amdgcn_global_load_lds(
+                        VTL_GPTR(EDGE ? pb[EDGE ? d - A_PW : 0] + ko : pb[0] + ko + (d - A_PW) * jstride),
+                        VTL_LPTR(sb_ + (w + NW * (d - A_PW)) * 1024), 16, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
     // scheduling hint: spread the TM+TN LDS reads of the next k-step between
     // the TM*TN MFMAs of the current one
     auto interleave = [&]() {
@@ -312,7 +342,9 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArg
     __builtin_amdgcn_s_barrier();
     lfrag(0, 0, 0);
     int st_c = 0;
-    for (int kt = 0; kt < KT - 1; kt++) {
+    // one tile but the last: k-steps 0..KS-2, hand-over, last k-step (with the
+    // loads of tile kt + NSTAGE between its MFMAs while there is such a tile)
+    auto tile_step = [&](auto with_issue, int kt) {
 #pragma unroll
         for (int s = 0; s < KS - 1; s++) {
             lfrag(st_c, s + 1, (s + 1) & 1);
@@ -323,18 +355,25 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArg
         // sure the next tile has landed, and hand this tile's buffer over
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         const int st_n = (st_c + 1 == NSTAGE) ? 0 : st_c + 1;
-        if (kt + NSTAGE - 1 < KT)
+        if (decltype(with_issue)::value || kt + NSTAGE - 1 < KT)
             wait_vmcnt<(NSTAGE - 2) * LPT>();
         else
             wait_vmcnt<0>();
         __builtin_amdgcn_s_barrier();
         lfrag(st_n, 0, 0);
-        mma((KS - 1) & 1);
-        if (kt + NSTAGE < KT)
-            issue(kt + NSTAGE, st_c);
-        interleave();
+        if constexpr (decltype(with_issue)::value) {
+            mma_issue((KS - 1) & 1, kt + NSTAGE, st_c);
+        } else {
+            mma((KS - 1) & 1);
+            interleave();
+        }
         st_c = st_n;
-    }
+    };
+    int kt = 0;
+    for (; kt + NSTAGE < KT; kt++)
+        tile_step(std::true_type{}, kt);
+    for (; kt < KT - 1; kt++)
+        tile_step(std::false_type{}, kt);
 #pragma unroll
     for (int s = 0; s < KS - 1; s++) {
         lfrag(st_c, s + 1, (s + 1) & 1);
