@@ -362,8 +362,10 @@ def bench_copy_calibration(timer: Timer, steps: int, warmup: int):
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    # the shader clock settles over the first tens of milliseconds of load: the
+    # defaults warm up for about that long and time a few hundred launches
+    ap.add_argument("--steps", type=int, default=300)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only", choices=["all", "linear", "quant", "copy", "full"], default="all")
     args = ap.parse_args()

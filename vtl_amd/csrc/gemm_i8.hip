@@ -287,35 +287,52 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArg
             for (int j = 0; j < TN; j++)
                 acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[buf][i], bf[buf][j], acc[i][j], 0, 0, 0);
     };
-    // The last k-step of a tile with the next tile's loads issued between its
-    // MFMAs, a few after each, in a fixed order.  Issued in one burst right
-    // after the barrier, the loads of all waves pile up in front of the compute
-    // unit's one address unit and the in-order waves stall behind them instead
-    // of issuing MFMAs.
-    auto mma_issue = [&](int buf, int kt, int st) {
-        constexpr int NM = TM * TN, PER = (LPT + NM - 1) / NM;  // loads after each MFMA
+    // One k-step in a fixed instruction order: MFMA q, then one operand read of
+    // the following k-step (stage rd_st, k-step rd_s, into register set rd_buf;
+    // A tiles first, then B), then this MFMA's share of the loads d0..d1-1 of
+    // tile `tile` into stage st.  Issued in one burst right after the barrier,
+    // the loads of all waves pile up in front of the compute unit's one address
+    // unit and the in-order waves stall behind them instead of issuing MFMAs.
+    auto step_fixed = [&](int buf, int rd_st, int rd_s, int rd_buf, int tile, int st, int d0, int d1) {
+        constexpr int NM = TM * TN, NR = TM + TN;
+        const int per = (d1 - d0 + NM - 1) / NM;  // loads after each MFMA
+        const char *rbase = smem + rd_st * STAGE;
         char *sa_ = smem + st * STAGE;
         char *sb_ = sa_ + BM * BK;
-        const int64_t ko = (int64_t)(kt_begin + kt) * BK;
+        const int64_t ko = (int64_t)(kt_begin + tile) * BK;
+        auto read_one = [&](int r) {
+            if (r < TM)
+                af[rd_buf][r] = *reinterpret_cast<const v4i *>(rbase + a_base + r * 32 * BK + foff[rd_s]);
+            else
+                bf[rd_buf][r - TM] =
+                    *reinterpret_cast<const v4i *>(rbase + b_base + (r - TM) * 32 * BK + foff[rd_s]);
+        };
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int q = 0; q < NM; q++) {
             acc[q / TN][q % TN] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[buf][q / TN], bf[buf][q % TN],
                                                                         acc[q / TN][q % TN], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
+            if (q < NR)
+                read_one(q);
 #pragma unroll
-            for (int d = q * PER; d < (q + 1) * PER && d < LPT; d++) {
-                if (d < A_PW)
-                    __builtin_amdgcn_global_load_lds(
-                        VTL_GPTR(EDGE ? pa[EDGE ? d : 0] + ko : pa[0] + ko + d * jstride),
-                        VTL_LPTR(sa_ + (w + NW * d) * 1024), 16, 0, 0);
-                else
-                    __builtin_amdgcn_global_load_lds(
-                        VTL_GPTR(EDGE ? pb[EDGE ? d - A_PW : 0] + ko : pb[0] + ko + (d - A_PW) * jstride),
-                        VTL_LPTR(sb_ + (w + NW * (d - A_PW)) * 1024), 16, 0, 0);
+            for (int d = 0; d < LPT; d++) {
+                if (d >= d0 + q * per && d < d0 + (q + 1) * per && d < d1) {
+                    if (d < A_PW)
+                        __builtin_amdgcn_global_load_lds(
+                            VTL_GPTR(EDGE ? pa[EDGE ? d : 0] + ko : pa[0] + ko + d * jstride),
+                            VTL_LPTR(sa_ + (w + NW * d) * 1024), 16, 0, 0);
+                    else
+                        __builtin_amdgcn_global_load_lds(
+                            VTL_GPTR(EDGE ? pb[EDGE ? d - A_PW : 0] + ko : pb[0] + ko + (d - A_PW) * jstride),
+                            VTL_LPTR(sb_ + (w + NW * (d - A_PW)) * 1024), 16, 0, 0);
+                }
             }
             __builtin_amdgcn_sched_barrier(0);
         }
+#pragma unroll
+        for (int r = NM; r < NR; r++)
+            read_one(r);
     };
     // scheduling hint: spread the TM+TN LDS reads of the next k-step between
     // the TM*TN MFMAs of the current one
@@ -342,14 +359,27 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArg
     __builtin_amdgcn_s_barrier();
     lfrag(0, 0, 0);
     int st_c = 0;
-    // one tile but the last: k-steps 0..KS-2, hand-over, last k-step (with the
-    // loads of tile kt + NSTAGE between its MFMAs while there is such a tile)
-    auto tile_step = [&](auto with_issue, int kt) {
+    // One tile but the last: k-steps 0..KS-2, hand-over, last k-step.  The
+    // stage that the hand-over of tile kt frees takes tile kt + NSTAGE; its
+    // loads are spread over SPREAD k-steps, the first share in the last k-step
+    // of tile kt (with_issue), the others in the first k-steps of tile kt + 1
+    // (with_prev, seen from that tile).  With two stages the tile is needed
+    // again one tile later, so everything goes into the one k-step; with more,
+    // three k-steps measured best (four delays the last share too much when the
+    // operands come from HBM, as in a split-K launch).
+    constexpr int SPREAD = NSTAGE >= 3 ? (KS < 3 ? KS : 3) : 1;
+    auto tile_step = [&](auto with_prev, auto with_issue, int kt) {
+        const int st_p = (st_c == 0) ? NSTAGE - 1 : st_c - 1;
 #pragma unroll
         for (int s = 0; s < KS - 1; s++) {
-            lfrag(st_c, s + 1, (s + 1) & 1);
-            mma(s & 1);
-            interleave();
+            if (decltype(with_prev)::value && s + 1 < SPREAD) {
+                step_fixed(s & 1, st_c, s + 1, (s + 1) & 1, kt - 1 + NSTAGE, st_p, (s + 1) * LPT / SPREAD,
+                           (s + 2) * LPT / SPREAD);
+            } else {
+                lfrag(st_c, s + 1, (s + 1) & 1);
+                mma(s & 1);
+                interleave();
+            }
         }
         // every operand read of this tile has been issued: wait for them, make
         // sure the next tile has landed, and hand this tile's buffer over
@@ -360,20 +390,29 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArg
         else
             wait_vmcnt<0>();
         __builtin_amdgcn_s_barrier();
-        lfrag(st_n, 0, 0);
         if constexpr (decltype(with_issue)::value) {
-            mma_issue((KS - 1) & 1, kt + NSTAGE, st_c);
+            step_fixed((KS - 1) & 1, st_n, 0, 0, kt + NSTAGE, st_c, 0, LPT / SPREAD);
         } else {
+            lfrag(st_n, 0, 0);
             mma((KS - 1) & 1);
             interleave();
         }
         st_c = st_n;
     };
+    using Yes = std::true_type;
+    using No = std::false_type;
+    using Prev = std::integral_constant<bool, (SPREAD > 1)>;
     int kt = 0;
-    for (; kt + NSTAGE < KT; kt++)
-        tile_step(std::true_type{}, kt);
+    if (NSTAGE < KT) {
+        tile_step(No{}, Yes{}, 0);
+        for (kt = 1; kt + NSTAGE < KT; kt++)
+            tile_step(Prev{}, Yes{}, kt);
+        // kt == KT - NSTAGE: the rest of the last tile's loads, no new tile
+        tile_step(Prev{}, No{}, kt);
+        kt++;
+    }
     for (; kt < KT - 1; kt++)
-        tile_step(std::false_type{}, kt);
+        tile_step(No{}, No{}, kt);
 #pragma unroll
     for (int s = 0; s < KS - 1; s++) {
         lfrag(st_c, s + 1, (s + 1) & 1);
@@ -1136,7 +1175,7 @@ struct TileConfig {
     int wgs_per_cu;     // workgroups that fit a compute unit's LDS together
 };
 constexpr TileConfig kTileConfigs[] = {
-    {32, 64, 330.f, 1}, {32, 128, 520.f, 2}, {64, 128, 640.f, 2}, {128, 128, 1150.f, 2}, {256, 256, 2600.f, 1}};
+    {32, 64, 330.f, 1}, {32, 128, 440.f, 2}, {64, 128, 560.f, 2}, {128, 128, 1075.f, 2}, {256, 256, 2400.f, 1}};
 constexpr int kNumTileConfigs = 5;
 
 template <bool F32OUT>
@@ -1173,8 +1212,8 @@ void choose_config(int M, int N, int K, int &best_idx, int &best_splits)
                 break;
             const int64_t rounds = (tiles * s + 256 * c.wgs_per_cu - 1) / (256 * c.wgs_per_cu);
             const int steps = (kt_all + s - 1) / s;
-            const float latency = (float)rounds * ((float)steps * c.step_cycles + 3000.f);
-            const float throughput = (float)tiles * (float)s * (float)steps * c.step_cycles / 256.f + 3000.f;
+            const float latency = (float)rounds * ((float)steps * c.step_cycles + 2000.f);
+            const float throughput = (float)tiles * (float)s * (float)steps * c.step_cycles / 256.f + 2000.f;
             float cost = latency > throughput ? latency : throughput;
             if (s > 1)
                 cost += 4500.f + (float)s * (float)M * (float)N * 4.0f / 2500.f;
