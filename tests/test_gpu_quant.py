@@ -165,6 +165,23 @@ def test_bit_pattern_sweep_against_oracle(hip):
         assert np.array_equal(got, ref), scale
 
 
+@pytest.mark.parametrize("scale", [3.7 / 127, 1e-39])
+def test_all_f32_bit_patterns_one_scale(hip, scale):
+    """All 2^32 f32 bit patterns through the quantizer with one scale (a normal
+    one that is no power of two; a subnormal one, which takes the kernel's
+    exact-division path), against the oracle's true division, in chunks of 2^27."""
+    sc = np.array([scale], np.float32)
+    chunk = 1 << 27
+    for c in range((1 << 32) // chunk):
+        x = np.arange(c * chunk, (c + 1) * chunk, dtype=np.uint64).astype(np.uint32).view(np.float32)
+        x = x.reshape(-1, 1 << 16)
+        got = _codes_with_scale(hip, x, sc)
+        ref = quantize_with_scale_mt(x, sc, False)
+        if not np.array_equal(got, ref):
+            bad = tuple(np.argwhere(got != ref)[0])
+            raise AssertionError((c, x[bad].view(np.uint32), got[bad], ref[bad]))
+
+
 def test_engineered_near_ties_per_row(hip):
     """Rows whose quotients sit within an ulp or two of k + 0.5."""
     rng = np.random.Generator(np.random.Philox(17))
