@@ -187,9 +187,10 @@ __device__ __forceinline__ void epilogue(v16i (&acc)[WM / 32][WN / 32], const Ge
 // (global_load_lds_dwordx4, no register staging): a wave instruction fills
 // 1 KiB of LDS in lane order, so the XOR swizzle is applied on the global side
 // (each lane fetches the chunk that belongs at its LDS slot).  NSTAGE tiles are
-// in flight.  MFMA operands are double-buffered in registers, and the
-// per-tile barrier sits before the last k-step of a tile so that its latency
-// and the first operand reads of the next tile hide behind that step's MFMAs.
+// in flight.  MFMA operands are double-buffered in registers, the per-tile
+// barrier sits before the last k-step of a tile so that its latency and the
+// first operand reads of the next tile hide behind that step's MFMAs, and the
+// loads that refill the freed stage are issued a few at a time between MFMAs.
 // Requires K % BK == 0; with EDGE, rows past M / N are clamped on load and
 // masked on store.
 template <int BM, int BN, int BK, int NSTAGE, int WR, int WC, bool F32OUT, bool EDGE, bool SPLIT>
@@ -290,9 +291,12 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArg
     // One k-step in a fixed instruction order: MFMA q, then one operand read of
     // the following k-step (stage rd_st, k-step rd_s, into register set rd_buf;
     // A tiles first, then B), then this MFMA's share of the loads d0..d1-1 of
-    // tile `tile` into stage st.  Issued in one burst right after the barrier,
-    // the loads of all waves pile up in front of the compute unit's one address
-    // unit and the in-order waves stall behind them instead of issuing MFMAs.
+    // tile `tile` into stage st.  Why the loads are handed out like this: when
+    // every wave issues all of its loads in one burst right after the barrier,
+    // they pile up in front of the compute unit's one address unit (16 cycles
+    // per wave instruction) and the in-order waves wait behind them instead of
+    // issuing MFMAs - measured 93.9 k against 83.5 k cycles for the K loop of
+    // the 256x256 tile at K = 4096.
     auto step_fixed = [&](int buf, int rd_st, int rd_s, int rd_buf, int tile, int st, int d0, int d1) {
         constexpr int NM = TM * TN, NR = TM + TN;
         const int per = (d1 - d0 + NM - 1) / NM;  // loads after each MFMA
