@@ -235,6 +235,79 @@ __global__ __launch_bounds__(T) void quantize_scaled_kernel(const float *__restr
     }
 }
 
+// Rows shorter than a workgroup's chunk (cols < 4 * T * NV, cols % 4 == 0): one
+// workgroup per row would leave most lanes idle (262144 rows of 256: 1.3 TB/s),
+// so the matrix is walked as one flat run of 16-byte vectors and every vector
+// looks up its row.  nvr = cols / 4.
+template <int T, int NV>
+__device__ __forceinline__ void short_rows_index(unsigned nvr, int64_t &base, int64_t &row0, unsigned &off0)
+{
+    base = (int64_t)blockIdx.x * (T * NV);
+    row0 = base / nvr;                       // uniform over the workgroup
+    off0 = (unsigned)(base - row0 * nvr);
+}
+
+template <int T, int NV>
+__global__ __launch_bounds__(T) void quantize_scaled_short_rows_kernel(const float *__restrict__ x,
+                                                                       const float *__restrict__ scale,
+                                                                       unsigned nvr, int64_t nv_total,
+                                                                       int8_t *__restrict__ q)
+{
+    int64_t base, row0;
+    unsigned off0;
+    short_rows_index<T, NV>(nvr, base, row0, off0);
+    const float4_t *xv = reinterpret_cast<const float4_t *>(x);
+    unsigned *qv = reinterpret_cast<unsigned *>(q);
+    float4_t v[NV];
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int64_t idx = base + i * T + threadIdx.x;
+        if (idx < nv_total)
+            v[i] = __builtin_nontemporal_load(xv + idx);
+    }
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int64_t idx = base + i * T + threadIdx.x;
+        if (idx < nv_total) {
+            const int64_t row = row0 + (off0 + (unsigned)(i * T) + threadIdx.x) / nvr;
+            __builtin_nontemporal_store(quant4(v[i], make_quant_scale(scale[row])), qv + idx);
+        }
+    }
+}
+
+template <int T, int NV>
+__global__ __launch_bounds__(T) void dequantize_short_rows_kernel(const int8_t *__restrict__ q,
+                                                                  const float *__restrict__ scale, unsigned nvr,
+                                                                  int64_t nv_total, float *__restrict__ x)
+{
+    int64_t base, row0;
+    unsigned off0;
+    short_rows_index<T, NV>(nvr, base, row0, off0);
+    const unsigned *qv = reinterpret_cast<const unsigned *>(q);
+    float4_t *xv = reinterpret_cast<float4_t *>(x);
+    unsigned c[NV];
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int64_t idx = base + i * T + threadIdx.x;
+        c[i] = (idx < nv_total) ? __builtin_nontemporal_load(qv + idx) : 0u;
+    }
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int64_t idx = base + i * T + threadIdx.x;
+        if (idx < nv_total) {
+            const int64_t row = row0 + (off0 + (unsigned)(i * T) + threadIdx.x) / nvr;
+            const float s = scale[row];
+            const unsigned w = c[i];
+            float4_t o;
+            o.x = (float)((int)(w << 24) >> 24) * s;
+            o.y = (float)((int)(w << 16) >> 24) * s;
+            o.z = (float)((int)(w << 8) >> 24) * s;
+            o.w = (float)((int)w >> 24) * s;
+            __builtin_nontemporal_store(o, xv + idx);
+        }
+    }
+}
+
 // ---- dequantize -------------------------------------------------------------
 
 // Same chunk-major block indexing as quantize_scaled_kernel.  Each lane reads four codes
@@ -459,6 +532,15 @@ int vtl_hip_quantize_with_scale_f32_i8(const float *x, const float *scale, int64
     const int64_t row_len = per_row ? cols : rows * cols;
     const bool vec = aligned(x, 16) && aligned(q, 4) && (!per_row || cols % 4 == 0);
     const int64_t per_chunk = vec ? 4 * T * NV : T * NV;
+    if (per_row && vec && rows > 1 && cols < per_chunk) {
+        const int64_t nv_total = rows * (cols >> 2);
+        const int64_t nblocks = (nv_total + T * NV - 1) / (T * NV);
+        if (nblocks > kMaxGridX)
+            return VTL_HIP_ERR_UNSUPPORTED;
+        hipLaunchKernelGGL((quantize_scaled_short_rows_kernel<T, NV>), dim3((unsigned)nblocks), dim3(T), 0, s, x,
+                           scale, (unsigned)(cols >> 2), nv_total, q);
+        return check_launch("quantize_scaled_short_rows_kernel");
+    }
     const int64_t chunks = (row_len + per_chunk - 1) / per_chunk;
     const int64_t blocks = per_row ? rows * chunks : chunks;
     if (chunks > kMaxGridX || blocks > kMaxGridX)
@@ -517,6 +599,15 @@ int vtl_hip_dequantize_i8_f32(const int8_t *q, const float *scale, int64_t rows,
     const int64_t row_len = per_row ? cols : rows * cols;
     const bool vec = aligned(x, 16) && aligned(q, 4) && (!per_row || cols % 4 == 0);
     const int64_t per_chunk = vec ? 4 * T * NV : T * NV;
+    if (per_row && vec && rows > 1 && cols < per_chunk) {
+        const int64_t nv_total = rows * (cols >> 2);
+        const int64_t nblocks = (nv_total + T * NV - 1) / (T * NV);
+        if (nblocks > kMaxGridX)
+            return VTL_HIP_ERR_UNSUPPORTED;
+        hipLaunchKernelGGL((dequantize_short_rows_kernel<T, NV>), dim3((unsigned)nblocks), dim3(T), 0, s, q, scale,
+                           (unsigned)(cols >> 2), nv_total, x);
+        return check_launch("dequantize_short_rows_kernel");
+    }
     const int64_t chunks = (row_len + per_chunk - 1) / per_chunk;
     const int64_t blocks = per_row ? rows * chunks : chunks;
     if (chunks > kMaxGridX || blocks > kMaxGridX)
