@@ -69,7 +69,9 @@ def test_row_quantize_known_answers(hip):
 SHAPES = [(1, 1), (1, 3), (7, 64), (5, 256), (3, 1000), (16, 784), (4, 4096), (2, 16384), (3, 16388),
           (2, 65536), (1, 70000), (3, 777), (2, 262148), (129, 12), (1000, 4), (64, 129),
           # short rows: workgroups span several rows, rows straddle workgroups
-          (5000, 1000), (70000, 8), (1025, 4092), (3000, 2052), (2, 4092)]
+          (5000, 1000), (70000, 8), (1025, 4092), (3000, 2052), (2, 4092),
+          # one row length per workgroup size of the fused kernel
+          (9, 512), (10, 2048), (6, 8192), (3, 5000), (5, 11008)]
 
 
 @pytest.mark.parametrize("shape", SHAPES)
