@@ -56,7 +56,9 @@ def test_maximum_k_accumulates_without_overflow(hip):
 
 SHAPES = [(1, 1, 16), (1, 64, 4096), (8, 128, 256), (33, 65, 48), (17, 19, 23), (64, 256, 784),
           (128, 128, 128), (256, 256, 128), (256, 512, 512), (300, 200, 144), (257, 255, 1040),
-          (512, 768, 384), (96, 11008 // 8, 640), (1024, 1024, 256), (5, 7, 1), (2, 3, 17)]
+          (512, 768, 384), (96, 11008 // 8, 640), (1024, 1024, 256), (5, 7, 1), (2, 3, 17),
+          # K a multiple of 16 but not of the 128-byte tile depth, on every tile size
+          (300, 300, 48), (40, 2100, 400), (64, 2100, 400), (130, 2100, 2000), (1100, 1100, 1936), (2100, 2100, 272)]
 
 
 @pytest.mark.parametrize("mnk", SHAPES)
@@ -190,9 +192,11 @@ def test_every_kernel_family_matches_oracle(hip, mnk):
         h.release()
 
 
-def test_forced_split_k_is_exact(hip, monkeypatch):
-    """Every tile configuration with 1, 2, 3 and 8 K ranges gives the same int32 result."""
-    m, n, k = 96, 384, 2432          # 19 K steps of 128: uneven ranges for every split count
+@pytest.mark.parametrize("k", [2432, 2448, 80])   # 19 K steps of 128; the same plus a 16-byte tail; one partial step
+def test_forced_split_k_is_exact(hip, monkeypatch, k):
+    """Every tile configuration with 1, 2, 3 and 8 K ranges gives the same int32 result
+    (uneven ranges for every split count)."""
+    m, n = 96, 384
     a, bt, sa, sb, bias = workloads.square_int8_gemm(m, n, k, seed=77)
     ref = oracle.gemm_i8_i32(a, bt, threads=CPU_THREADS)
     want = oracle.epilogue(ref, sa, sb, bias)

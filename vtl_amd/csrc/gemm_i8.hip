@@ -183,6 +183,9 @@ __device__ __forceinline__ void epilogue(v16i (&acc)[WM / 32][WN / 32], const Ge
     }
 }
 
+// Sixteen zero bytes in device memory: what lanes past the end of K load.
+__device__ __attribute__((aligned(16))) int8_t g_zero_chunk[16];
+
 // Main kernel.  Operand tiles go from global memory straight into LDS
 // (global_load_lds_dwordx4, no register staging): a wave instruction fills
 // 1 KiB of LDS in lane order, so the XOR swizzle is applied on the global side
@@ -191,8 +194,9 @@ __device__ __forceinline__ void epilogue(v16i (&acc)[WM / 32][WN / 32], const Ge
 // barrier sits before the last k-step of a tile so that its latency and the
 // first operand reads of the next tile hide behind that step's MFMAs, and the
 // loads that refill the freed stage are issued a few at a time between MFMAs.
-// Requires K % BK == 0; with EDGE, rows past M / N are clamped on load and
-// masked on store.
+// Requires K % BK == 0, or with EDGE K % 16 == 0: then the chunks of the last
+// tile that lie past K are loaded as zeros, rows past M / N are clamped on load
+// and masked on store.
 template <int BM, int BN, int BK, int NSTAGE, int WR, int WC, bool F32OUT, bool EDGE, bool SPLIT>
 __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArgs g)
 {
@@ -219,7 +223,7 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArg
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int wr = w / WC, wc = w % WC;
-    const int kt_all = K / BK;
+    const int kt_all = EDGE ? (K + BK - 1) / BK : K / BK;  // EDGE: the last tile may be partial in K
     const int kt_begin = SPLIT ? (int)((int64_t)kt_all * split / nsplit) : 0;
     const int kt_end = SPLIT ? (int)((int64_t)kt_all * (split + 1) / nsplit) : kt_all;
 
@@ -240,18 +244,32 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArg
         pb[0] = g.Bt + (int64_t)(n0 + lrow) * K + lc * 16;
     }
     const int64_t jstride = (int64_t)RPI * NW * K;
+    // Global source of load d (A rows first, then B) of the tile at K offset ko.
+    // With EDGE, a lane whose 16-byte chunk lies past K reads zeros instead
+    // (K % 16 == 0, so a chunk is inside or outside as a whole).
+    auto source = [&](int d, int64_t ko) -> const int8_t * {
+        const int8_t *p;
+        if (d < A_PW)
+            p = EDGE ? pa[EDGE ? d : 0] + ko : pa[0] + ko + d * jstride;
+        else
+            p = EDGE ? pb[EDGE ? d - A_PW : 0] + ko : pb[0] + ko + (d - A_PW) * jstride;
+        if constexpr (EDGE) {
+            if (ko + lc * 16 >= K)
+                p = g_zero_chunk;
+        }
+        return p;
+    };
     auto issue = [&](int kt, int st) {
         char *sa_ = smem + st * STAGE;
         char *sb_ = sa_ + BM * BK;
         const int64_t ko = (int64_t)(kt_begin + kt) * BK;
 #pragma unroll
         for (int j = 0; j < A_PW; j++)
-            __builtin_amdgcn_global_load_lds(VTL_GPTR(EDGE ? pa[EDGE ? j : 0] + ko : pa[0] + ko + j * jstride),
-                                             VTL_LPTR(sa_ + (w + NW * j) * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(VTL_GPTR(source(j, ko)), VTL_LPTR(sa_ + (w + NW * j) * 1024), 16, 0, 0);
 #pragma unroll
         for (int j = 0; j < B_PW; j++)
-            __builtin_amdgcn_global_load_lds(VTL_GPTR(EDGE ? pb[EDGE ? j : 0] + ko : pb[0] + ko + j * jstride),
-                                             VTL_LPTR(sb_ + (w + NW * j) * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(VTL_GPTR(source(A_PW + j, ko)), VTL_LPTR(sb_ + (w + NW * j) * 1024), 16,
+                                             0, 0);
     };
 
     v16i acc[TM][TN];
@@ -323,13 +341,11 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArg
             for (int d = 0; d < LPT; d++) {
                 if (d >= d0 + q * per && d < d0 + (q + 1) * per && d < d1) {
                     if (d < A_PW)
-                        __builtin_amdgcn_global_load_lds(
-                            VTL_GPTR(EDGE ? pa[EDGE ? d : 0] + ko : pa[0] + ko + d * jstride),
-                            VTL_LPTR(sa_ + (w + NW * d) * 1024), 16, 0, 0);
+                        __builtin_amdgcn_global_load_lds(VTL_GPTR(source(d, ko)),
+                                                         VTL_LPTR(sa_ + (w + NW * d) * 1024), 16, 0, 0);
                     else
-                        __builtin_amdgcn_global_load_lds(
-                            VTL_GPTR(EDGE ? pb[EDGE ? d - A_PW : 0] + ko : pb[0] + ko + (d - A_PW) * jstride),
-                            VTL_LPTR(sb_ + (w + NW * (d - A_PW)) * 1024), 16, 0, 0);
+                        __builtin_amdgcn_global_load_lds(VTL_GPTR(source(d, ko)),
+                                                         VTL_LPTR(sb_ + (w + NW * (d - A_PW)) * 1024), 16, 0, 0);
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -885,108 +901,6 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_skinny_dynquant_kernel(cons
     }
 }
 
-// Register-staged tile kernel for K that is a multiple of 16 but not of the
-// DMA kernel's tile depth: global -> VGPR -> LDS, zero-filled K tail.
-template <int BM, int BN, int WR, int WC, bool F32OUT>
-__global__ __launch_bounds__(64 * WR * WC) void gemm_i8_tile_kernel(const GemmArgs g)
-{
-    constexpr int BK = 128;
-    constexpr int NT = 64 * WR * WC;
-    constexpr int WM = BM / WR, WN = BN / WC;
-    constexpr int TM = WM / 32, TN = WN / 32;
-    constexpr int A_CH = BM * 8 / NT, B_CH = BN * 8 / NT;
-    constexpr int ROWS_PER_PASS = NT / 8;
-    static_assert(BM % (32 * WR) == 0 && BN % (32 * WC) == 0, "wave tile must be a multiple of 32");
-    static_assert(A_CH >= 1 && B_CH >= 1 && (BM * 8) % NT == 0 && (BN * 8) % NT == 0, "copy split");
-
-    extern __shared__ __attribute__((aligned(16))) char smem[];
-    char *sA = smem;                // [2][BM * BK]
-    char *sB = smem + 2 * BM * BK;  // [2][BN * BK]
-
-    const int M = g.M, N = g.N, K = g.K;
-    int tile_m, tile_n;
-    tile_of_block((M + BM - 1) / BM, (N + BN - 1) / BN, (int)blockIdx.x, tile_m, tile_n);
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wr = wave / WC, wc = wave % WC;
-
-    const int cc = tid & 7;   // 16-byte chunk inside the 128-byte row
-    const int cr = tid >> 3;  // first row this thread copies
-    v4i ra[A_CH], rb[B_CH];
-    auto gload = [&](int kt) {
-        const int kbyte = kt * BK + cc * 16;
-#pragma unroll
-        for (int i = 0; i < A_CH; i++) {
-            const int row = min(m0 + cr + i * ROWS_PER_PASS, M - 1);
-            const v4i *p = reinterpret_cast<const v4i *>(g.A + (int64_t)row * K + kbyte);
-            ra[i] = (kbyte < K) ? *p : v4i{0, 0, 0, 0};
-        }
-#pragma unroll
-        for (int i = 0; i < B_CH; i++) {
-            const int row = min(n0 + cr + i * ROWS_PER_PASS, N - 1);
-            const v4i *p = reinterpret_cast<const v4i *>(g.Bt + (int64_t)row * K + kbyte);
-            rb[i] = (kbyte < K) ? *p : v4i{0, 0, 0, 0};
-        }
-    };
-    auto lstore = [&](int buf) {
-        char *a = sA + buf * (BM * BK);
-        char *b = sB + buf * (BN * BK);
-#pragma unroll
-        for (int i = 0; i < A_CH; i++)
-            *reinterpret_cast<v4i *>(a + lds_off<BK>(cr + i * ROWS_PER_PASS, cc)) = ra[i];
-#pragma unroll
-        for (int i = 0; i < B_CH; i++)
-            *reinterpret_cast<v4i *>(b + lds_off<BK>(cr + i * ROWS_PER_PASS, cc)) = rb[i];
-    };
-
-    v16i acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; i++)
-#pragma unroll
-        for (int j = 0; j < TN; j++)
-#pragma unroll
-            for (int r = 0; r < 16; r++)
-                acc[i][j][r] = 0;
-
-    const int frow = lane & 31;
-    const int fch = lane >> 5;
-    auto compute = [&](int buf) {
-        const char *a = sA + buf * (BM * BK);
-        const char *b = sB + buf * (BN * BK);
-#pragma unroll
-        for (int s = 0; s < BK / 32; s++) {
-            v4i af[TM], bf[TN];
-            const int ch = s * 2 + fch;
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-                af[i] = *reinterpret_cast<const v4i *>(a + lds_off<BK>(wr * WM + i * 32 + frow, ch));
-#pragma unroll
-            for (int j = 0; j < TN; j++)
-                bf[j] = *reinterpret_cast<const v4i *>(b + lds_off<BK>(wc * WN + j * 32 + frow, ch));
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int j = 0; j < TN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
-        }
-    };
-
-    const int KT = (K + BK - 1) / BK;
-    gload(0);
-    lstore(0);
-    __syncthreads();
-    for (int kt = 0; kt < KT; kt++) {
-        const bool more = kt + 1 < KT;
-        if (more)
-            gload(kt + 1);
-        compute(kt & 1);
-        if (more)
-            lstore((kt + 1) & 1);
-        __syncthreads();
-    }
-    epilogue<BM, BN, WM, WN, F32OUT, true, NT>(acc, g, m0, n0, wr, wc, smem);
-}
-
 // Any shape, any alignment: one output per thread.  Only used when K is not a
 // multiple of 16 or a pointer is not 16-byte aligned.
 template <bool F32OUT>
@@ -1119,7 +1033,7 @@ int launch_dma(GemmArgs g, int splits, hipStream_t st)
     static_assert(lds >= (BM + 2 * BN) * 4, "epilogue staging fits in the operand buffers");
     static_assert((NSTAGE - 1) * ((BM + BN) / (64 / (BK / 16)) / (WR * WC)) <= 63, "vmcnt is a 6-bit counter");
     const int tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
-    const int kt_all = g.K / BK;
+    const int kt_all = (g.K + BK - 1) / BK;
     if (splits > kt_all)
         splits = kt_all;
     if (splits < 1)
@@ -1133,7 +1047,7 @@ int launch_dma(GemmArgs g, int splits, hipStream_t st)
     }
     static PerDevice<bool> done_flags[4];
     bool *done[4] = {&done_flags[0].get(), &done_flags[1].get(), &done_flags[2].get(), &done_flags[3].get()};
-    const bool edge = (g.M % BM) || (g.N % BN);
+    const bool edge = (g.M % BM) || (g.N % BN) || (g.K % BK);
     int rc;
     // the partial sums of a split launch are int32 whatever the final type is
     if (splits > 1 && edge)
@@ -1159,17 +1073,6 @@ int launch_dma(GemmArgs g, int splits, hipStream_t st)
                            g);
     }
     return check_launch("splitk_finalize_kernel");
-}
-
-template <int BM, int BN, int WR, int WC, bool F32OUT>
-int launch_tile(const GemmArgs &g, hipStream_t st)
-{
-    constexpr int lds = 2 * (BM + BN) * 128;
-    const int tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
-    static PerDevice<bool> done_flag;
-    bool &done = done_flag.get();
-    return launch_with_lds(gemm_i8_tile_kernel<BM, BN, WR, WC, F32OUT>, done, lds, tiles, 64 * WR * WC, g, st,
-                           "gemm_i8_tile_kernel");
 }
 
 // The DMA-kernel instantiations, smallest tile first.
@@ -1206,7 +1109,7 @@ int launch_config(int idx, const GemmArgs &g, int splits, hipStream_t st)
 // exhaustive timing sweep of every tile and split count over 39 shapes.
 void choose_config(int M, int N, int K, int &best_idx, int &best_splits)
 {
-    const int kt_all = K / 128;
+    const int kt_all = (K + 127) / 128;
     float best = 3.0e38f;
     best_idx = kNumTileConfigs - 1;
     best_splits = 1;
@@ -1294,24 +1197,16 @@ int launch_gemm(const GemmArgs &g, hipStream_t st)
         hipLaunchKernelGGL((gemm_i8_small_kernel<F32OUT>), dim3((unsigned)t32), dim3(256), 0, st, g);
         return check_launch("gemm_i8_small_kernel");
     }
-    if (g.K % 128 == 0) {
-        int idx, splits;
-        choose_config(g.M, g.N, g.K, idx, splits);
-        if (const char *force = getenv("VTL_HIP_GEMM_CONFIG")) {  // tuning knob: "<tile index>,<splits>"
-            int fi = -1, fs = 1;
-            if (sscanf(force, "%d,%d", &fi, &fs) >= 1 && fi >= 0 && fi < kNumTileConfigs) {
-                idx = fi;
-                splits = fs;
-            }
+    int idx, splits;
+    choose_config(g.M, g.N, g.K, idx, splits);
+    if (const char *force = getenv("VTL_HIP_GEMM_CONFIG")) {  // tuning knob: "<tile index>,<splits>"
+        int fi = -1, fs = 1;
+        if (sscanf(force, "%d,%d", &fi, &fs) >= 1 && fi >= 0 && fi < kNumTileConfigs) {
+            idx = fi;
+            splits = fs;
         }
-        return launch_config<F32OUT>(idx, g, splits, st);
     }
-    const int64_t t128 = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
-    if (g.M > 64 && t128 >= 64)
-        return launch_tile<128, 128, 2, 2, F32OUT>(g, st);
-    if (g.M > 32)
-        return launch_tile<64, 64, 2, 2, F32OUT>(g, st);
-    return launch_tile<32, 64, 1, 2, F32OUT>(g, st);
+    return launch_config<F32OUT>(idx, g, splits, st);
 }
 
 int check_gemm_args(const void *A, const void *Bt, const void *out, int M, int N, int K)
