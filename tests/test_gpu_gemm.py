@@ -95,6 +95,31 @@ def test_unaligned_operands_take_the_generic_kernel(hip):
         h.release()
 
 
+@pytest.mark.parametrize("mnk", [(300, 200, 1000), (8, 2048, 4090), (64, 256, 777), (1100, 520, 2001),
+                                 (256, 1024, 1024), (20, 2304, 512)])
+def test_odd_k_and_unaligned_operands_are_repacked(hip, mnk):
+    """K that is no multiple of 16, and operands / outputs at odd addresses: the
+    library pads the rows into its own scratch and runs the fast kernels; results
+    are the oracle's bit for bit (int32 and the f32 epilogue)."""
+    m, n, k = mnk
+    a, bt, sa, sb, bias = workloads.square_int8_gemm(m, n, k, seed=m + n + k)
+    ref = oracle.gemm_i8_i32(a, bt, threads=CPU_THREADS)
+    want = oracle.epilogue(ref, sa, sb, bias, relu=True)
+    abuf, bbuf = raw_device_buffer(a.size + 64), raw_device_buffer(bt.size + 64)
+    cbuf, ybuf = raw_device_buffer(m * n * 4 + 64), raw_device_buffer(m * n * 4 + 64)
+    dsa, dsb, dbias = dev(sa), dev(sb), dev(bias)
+    for off_a, off_b, off_c in ((0, 0, 0), (3, 5, 4), (16, 1, 12)):
+        h2d(abuf.ptr + off_a, a)
+        h2d(bbuf.ptr + off_b, bt)
+        capi.call("vtl_hip_gemm_i8_i32", abuf.ptr + off_a, bbuf.ptr + off_b, cbuf.ptr + off_c, m, n, k)
+        assert np.array_equal(d2h(cbuf.ptr + off_c, (m, n), np.int32), ref), (off_a, off_b, off_c)
+        capi.call("vtl_hip_linear_i8_f32", abuf.ptr + off_a, dsa.ptr, 1, bbuf.ptr + off_b, dsb.ptr, 1, dbias.ptr,
+                  ybuf.ptr + off_c, m, n, k, 1)
+        assert np.array_equal(d2h(ybuf.ptr + off_c, (m, n), np.float32), want), (off_a, off_b, off_c)
+    for h in (abuf, bbuf, cbuf, ybuf, dsa, dsb, dbias):
+        h.release()
+
+
 def test_shape_mismatch_is_reported_like_la_matmul(hip):
     A, B = dev(np.zeros((4, 32), np.int8)), dev(np.zeros((6, 48), np.int8))
     Cm = HipTensor.empty([4, 6], np.int32)

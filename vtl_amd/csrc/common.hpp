@@ -21,9 +21,10 @@ int check_launch(const char *kernel_name);
 // Streaming copy kernel (quant.hip); false when alignment or size do not qualify.
 bool launch_copy(void *dst, const void *src, size_t bytes, hipStream_t st);
 
-// Device scratch owned by the library: per device two independent buffers
+// Device scratch owned by the library: per device three independent buffers
 // (slot 0: split-K partial sums and partial column sums; slot 1: quantized
-// activations staged between the two launches of a dynamic-quantization call),
+// activations staged between the two launches of a dynamic-quantization call;
+// slot 2: int8 operands repacked to a row length the fast kernels take),
 // grown on demand and kept until the process ends.  Kernels enqueued on the
 // current stream may use a slot until the next call that asks for it; nullptr
 // when the allocation fails.

@@ -929,6 +929,26 @@ __global__ __launch_bounds__(256) void gemm_i8_naive_kernel(const GemmArgs g)
     }
 }
 
+// Copies `rows` rows of K bytes into rows of Kp >= K bytes (Kp % 4 == 0), zero
+// filled: four destination bytes per thread.
+__global__ __launch_bounds__(256) void pad_rows_i8_kernel(const int8_t *__restrict__ src, int64_t rows, int K,
+                                                         int8_t *__restrict__ dst, int Kp)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int q = Kp >> 2;
+    if (i >= rows * q)
+        return;
+    const int64_t row = i / q;
+    const int c = (int)(i - row * q) * 4;
+    const int8_t *s = src + row * K;
+    unsigned w = 0;
+#pragma unroll
+    for (int b = 0; b < 4; b++)
+        if (c + b < K)
+            w |= (unsigned)(uint8_t)s[c + b] << (8 * b);
+    reinterpret_cast<unsigned *>(dst)[i] = w;
+}
+
 // Small products (a few dozen 32x32 output tiles): nothing is reused often
 // enough to stage, so each wave feeds the MFMA straight from global memory.
 // One workgroup per 32x32 tile; its four waves split the K steps and the
@@ -1180,14 +1200,39 @@ int launch_skinny_dynquant(const GemmArgs &g, hipStream_t st)
 }
 
 template <bool F32OUT>
-int launch_gemm(const GemmArgs &g, hipStream_t st)
+int launch_gemm(const GemmArgs &g_in, hipStream_t st)
 {
+    GemmArgs g = g_in;
     if ((g.K % 16) || !aligned16(g.A) || !aligned16(g.Bt)) {
+        // The fast kernels read 16-byte chunks of rows that start 16-byte
+        // aligned.  A tiny product is done one output per thread; anything
+        // else is first copied into zero-padded rows of the library's scratch
+        // (one more pass over the int8 operands: e.g. 1024x4096x4090 takes
+        // 21 ms output-per-thread and well under 0.1 ms this way).
         const dim3 grid((unsigned)((g.N + 15) / 16), (unsigned)((g.M + 15) / 16));
-        if (grid.y > 65535)
+        if ((int64_t)g.M * g.N * g.K <= (int64_t)1 << 20 && grid.y <= 65535) {
+            hipLaunchKernelGGL((gemm_i8_naive_kernel<F32OUT>), grid, dim3(256), 0, st, g);
+            return check_launch("gemm_i8_naive_kernel");
+        }
+        const int Kp = (g.K + 15) & ~15;
+        const size_t a_bytes = ((size_t)g.M * Kp + 255) & ~(size_t)255;
+        const size_t b_bytes = (size_t)g.N * Kp;
+        int8_t *ws = static_cast<int8_t *>(vtlhip::library_workspace(a_bytes + b_bytes, 2));
+        if (!ws)
+            return VTL_HIP_ERR_OUT_OF_MEMORY;
+        const int64_t ta = (int64_t)g.M * (Kp / 4), tb = (int64_t)g.N * (Kp / 4);
+        if ((ta + 255) / 256 > 0x7fffffff || (tb + 255) / 256 > 0x7fffffff)
             return VTL_HIP_ERR_UNSUPPORTED;
-        hipLaunchKernelGGL((gemm_i8_naive_kernel<F32OUT>), grid, dim3(256), 0, st, g);
-        return check_launch("gemm_i8_naive_kernel");
+        hipLaunchKernelGGL(pad_rows_i8_kernel, dim3((unsigned)((ta + 255) / 256)), dim3(256), 0, st, g.A,
+                           (int64_t)g.M, g.K, ws, Kp);
+        hipLaunchKernelGGL(pad_rows_i8_kernel, dim3((unsigned)((tb + 255) / 256)), dim3(256), 0, st, g.Bt,
+                           (int64_t)g.N, g.K, ws + a_bytes, Kp);
+        const int rc = check_launch("pad_rows_i8_kernel");
+        if (rc != VTL_HIP_OK)
+            return rc;
+        g.A = ws;
+        g.Bt = ws + a_bytes;
+        g.K = Kp;
     }
     if (g.K % 256 == 0 && g.M <= 32 && g.N >= 2048 && !getenv("VTL_HIP_GEMM_CONFIG"))
         return launch_skinny<F32OUT>(g, st);  // weight streaming: enough row blocks to fill the chip

@@ -36,9 +36,9 @@ int check_launch(const char *kernel_name)
 void *library_workspace(size_t bytes, int slot)
 {
     constexpr int kMaxDevices = 64;
-    static void *bufs[2][kMaxDevices] = {};
-    static size_t caps[2][kMaxDevices] = {};
-    if (slot < 0 || slot > 1)
+    static void *bufs[3][kMaxDevices] = {};
+    static size_t caps[3][kMaxDevices] = {};
+    if (slot < 0 || slot > 2)
         return nullptr;
     void **buf = bufs[slot];
     size_t *cap = caps[slot];
