@@ -21,6 +21,15 @@ namespace {
 
 using namespace vtlhip::qdev;
 
+// Elements of a row that starts at flat element `start` before the next
+// multiple of four (where 16-byte loads of f32 and 4-byte stores of codes are
+// aligned, the base pointers being aligned), at most the whole row.
+__device__ __forceinline__ int row_head(int64_t start, int64_t cols)
+{
+    const int h = (int)((4 - (start & 3)) & 3);
+    return h < cols ? h : (int)cols;
+}
+
 // ---- absmax ----------------------------------------------------------------
 
 // One workgroup per row, strided loop over the row.
@@ -33,8 +42,15 @@ __global__ __launch_bounds__(T) void absmax_rows_kernel(const float *__restrict_
     const float *xr = x + row * cols;
     float m = 0.0f;
     if constexpr (VEC == 4) {
-        const float4_t *xv = reinterpret_cast<const float4_t *>(xr);
-        const int64_t nv = cols >> 2;
+        // x is 16-byte aligned; a row of any length starts at most three
+        // elements before a 16-byte boundary: scalar head, vector body, scalar tail
+        const int head = row_head(row * cols, cols);
+        const float4_t *xv = reinterpret_cast<const float4_t *>(xr + head);
+        const int64_t nv = (cols - head) >> 2;
+        if ((int)threadIdx.x < head)
+            m = fabsf(xr[threadIdx.x]);
+        if ((int)threadIdx.x < (int)((cols - head) & 3))
+            m = fmaxf(m, fabsf(xr[head + (nv << 2) + threadIdx.x]));
         int64_t i = threadIdx.x;
         for (; i + 3 * T < nv; i += 4 * T) {  // four independent loads in flight per lane
             const float4_t v0 = __builtin_nontemporal_load(xv + i);
@@ -146,7 +162,7 @@ __global__ __launch_bounds__(T) void quantize_rows_reg_kernel(const float *__res
 }
 
 // Rows too long for registers, or not a multiple of four: two passes over the
-// row inside one workgroup (the second pass mostly hits L2 / MALL).
+// row inside one workgroup (the second pass mostly hits L2 / MALL).  T >= 4.
 template <int T, int VEC>
 __global__ __launch_bounds__(T) void quantize_rows_loop_kernel(const float *__restrict__ x,
                                                                int64_t cols, int8_t *__restrict__ q,
@@ -157,9 +173,17 @@ __global__ __launch_bounds__(T) void quantize_rows_loop_kernel(const float *__re
     const float *xr = x + row * cols;
     int8_t *qr = q + row * cols;
     float m = 0.0f;
+    // VEC == 4: x is 16-byte and q 4-byte aligned; scalar head up to the next
+    // multiple of four of the flat index, vector body, scalar tail
+    const int head = VEC == 4 ? row_head(row * cols, cols) : 0;
+    const int64_t nv = (cols - head) >> 2;
+    const int tail = (int)((cols - head) & 3);
     if constexpr (VEC == 4) {
-        const float4_t *xv = reinterpret_cast<const float4_t *>(xr);
-        const int64_t nv = cols >> 2;
+        const float4_t *xv = reinterpret_cast<const float4_t *>(xr + head);
+        if ((int)threadIdx.x < head)
+            m = fabsf(xr[threadIdx.x]);
+        if ((int)threadIdx.x < tail)
+            m = fmaxf(m, fabsf(xr[head + (nv << 2) + threadIdx.x]));
         for (int64_t i = threadIdx.x; i < nv; i += T)
             m = absmax4(m, xv[i]);
     } else {
@@ -172,9 +196,14 @@ __global__ __launch_bounds__(T) void quantize_rows_loop_kernel(const float *__re
         scale_out[row] = scale;
     const QuantScale p = make_quant_scale(scale);
     if constexpr (VEC == 4) {
-        const float4_t *xv = reinterpret_cast<const float4_t *>(xr);
-        unsigned *qv = reinterpret_cast<unsigned *>(qr);
-        const int64_t nv = cols >> 2;
+        const float4_t *xv = reinterpret_cast<const float4_t *>(xr + head);
+        unsigned *qv = reinterpret_cast<unsigned *>(qr + head);
+        if ((int)threadIdx.x < head)
+            qr[threadIdx.x] = (int8_t)quant_code(xr[threadIdx.x], p);
+        if ((int)threadIdx.x < tail) {
+            const int64_t i = head + (nv << 2) + threadIdx.x;
+            qr[i] = (int8_t)quant_code(xr[i], p);
+        }
         for (int64_t i = threadIdx.x; i < nv; i += T)
             qv[i] = quant4(xv[i], p);
     } else {
@@ -235,76 +264,122 @@ __global__ __launch_bounds__(T) void quantize_scaled_kernel(const float *__restr
     }
 }
 
-// Rows shorter than a workgroup's chunk (cols < 4 * T * NV, cols % 4 == 0): one
-// workgroup per row would leave most lanes idle (262144 rows of 256: 1.3 TB/s),
-// so the matrix is walked as one flat run of 16-byte vectors and every vector
-// looks up its row.  nvr = cols / 4.
+// Per-row scales over a matrix walked as ONE flat run of 16-byte vectors, each
+// element looking up its row: for rows shorter than a workgroup's chunk (one
+// workgroup per row would leave most lanes idle: 262144 rows of 256 ran at
+// 1.3 TB/s) and for row lengths that are no multiple of four (rows then start
+// at any alignment, the flat run does not).  cols >= 4, so a vector touches at
+// most two rows.  The workgroup divides once in 64 bits, its lanes in 32.
+struct FlatRows {
+    int64_t base;   // first vector of the workgroup
+    int64_t row_b;  // row of its first element
+    unsigned off_b; // column of its first element
+};
+
 template <int T, int NV>
-__device__ __forceinline__ void short_rows_index(unsigned nvr, int64_t &base, int64_t &row0, unsigned &off0)
+__device__ __forceinline__ FlatRows flat_rows_origin(unsigned cols)
 {
-    base = (int64_t)blockIdx.x * (T * NV);
-    row0 = base / nvr;                       // uniform over the workgroup
-    off0 = (unsigned)(base - row0 * nvr);
+    FlatRows f;
+    f.base = (int64_t)blockIdx.x * (T * NV);
+    const int64_t e = f.base << 2;
+    f.row_b = e / cols;
+    f.off_b = (unsigned)(e - f.row_b * cols);
+    return f;
+}
+
+// Row and column of the first element of vector `local` of the workgroup.
+__device__ __forceinline__ void flat_rows_locate(const FlatRows &f, unsigned cols, unsigned local, int64_t &row,
+                                                 unsigned &col)
+{
+    const unsigned e = f.off_b + 4u * local;
+    const unsigned r = e / cols;
+    row = f.row_b + r;
+    col = e - r * cols;
 }
 
 template <int T, int NV>
-__global__ __launch_bounds__(T) void quantize_scaled_short_rows_kernel(const float *__restrict__ x,
-                                                                       const float *__restrict__ scale,
-                                                                       unsigned nvr, int64_t nv_total,
-                                                                       int8_t *__restrict__ q)
+__global__ __launch_bounds__(T) void quantize_scaled_flat_rows_kernel(const float *__restrict__ x,
+                                                                      const float *__restrict__ scale,
+                                                                      unsigned cols, int64_t n,
+                                                                      int8_t *__restrict__ q)
 {
-    int64_t base, row0;
-    unsigned off0;
-    short_rows_index<T, NV>(nvr, base, row0, off0);
+    const FlatRows f = flat_rows_origin<T, NV>(cols);
+    const int64_t nv_total = n >> 2;
     const float4_t *xv = reinterpret_cast<const float4_t *>(x);
     unsigned *qv = reinterpret_cast<unsigned *>(q);
     float4_t v[NV];
 #pragma unroll
     for (int i = 0; i < NV; i++) {
-        const int64_t idx = base + i * T + threadIdx.x;
+        const int64_t idx = f.base + i * T + threadIdx.x;
         if (idx < nv_total)
             v[i] = __builtin_nontemporal_load(xv + idx);
     }
 #pragma unroll
     for (int i = 0; i < NV; i++) {
-        const int64_t idx = base + i * T + threadIdx.x;
+        const int64_t idx = f.base + i * T + threadIdx.x;
         if (idx < nv_total) {
-            const int64_t row = row0 + (off0 + (unsigned)(i * T) + threadIdx.x) / nvr;
-            __builtin_nontemporal_store(quant4(v[i], make_quant_scale(scale[row])), qv + idx);
+            int64_t row;
+            unsigned col;
+            flat_rows_locate(f, cols, (unsigned)(i * T) + threadIdx.x, row, col);
+            const QuantScale p = make_quant_scale(scale[row]);
+            unsigned packed;
+            if (col + 4 <= cols) {
+                packed = quant4(v[i], p);
+            } else {  // the vector runs into the next row
+                const QuantScale p1 = make_quant_scale(scale[row + 1]);
+                const unsigned in0 = cols - col;  // 1..3 elements still in `row`
+                packed = 0;
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    packed |= (unsigned)(uint8_t)(int8_t)quant_code(v[i][e], (unsigned)e < in0 ? p : p1) << (8 * e);
+            }
+            __builtin_nontemporal_store(packed, qv + idx);
         }
+    }
+    // the last n % 4 elements of the matrix belong to its last row
+    if (blockIdx.x == 0 && threadIdx.x < (unsigned)(n & 3)) {
+        const int64_t i = (nv_total << 2) + threadIdx.x;
+        q[i] = (int8_t)quant_code(x[i], make_quant_scale(scale[(n - 1) / cols]));
     }
 }
 
 template <int T, int NV>
-__global__ __launch_bounds__(T) void dequantize_short_rows_kernel(const int8_t *__restrict__ q,
-                                                                  const float *__restrict__ scale, unsigned nvr,
-                                                                  int64_t nv_total, float *__restrict__ x)
+__global__ __launch_bounds__(T) void dequantize_flat_rows_kernel(const int8_t *__restrict__ q,
+                                                                 const float *__restrict__ scale, unsigned cols,
+                                                                 int64_t n, float *__restrict__ x)
 {
-    int64_t base, row0;
-    unsigned off0;
-    short_rows_index<T, NV>(nvr, base, row0, off0);
+    const FlatRows f = flat_rows_origin<T, NV>(cols);
+    const int64_t nv_total = n >> 2;
     const unsigned *qv = reinterpret_cast<const unsigned *>(q);
     float4_t *xv = reinterpret_cast<float4_t *>(x);
     unsigned c[NV];
 #pragma unroll
     for (int i = 0; i < NV; i++) {
-        const int64_t idx = base + i * T + threadIdx.x;
+        const int64_t idx = f.base + i * T + threadIdx.x;
         c[i] = (idx < nv_total) ? __builtin_nontemporal_load(qv + idx) : 0u;
     }
 #pragma unroll
     for (int i = 0; i < NV; i++) {
-        const int64_t idx = base + i * T + threadIdx.x;
+        const int64_t idx = f.base + i * T + threadIdx.x;
         if (idx < nv_total) {
-            const int64_t row = row0 + (off0 + (unsigned)(i * T) + threadIdx.x) / nvr;
-            const float s = scale[row];
+            int64_t row;
+            unsigned col;
+            flat_rows_locate(f, cols, (unsigned)(i * T) + threadIdx.x, row, col);
+            const float s0 = scale[row];
+            const unsigned in0 = cols - col;  // elements of the vector still in `row` (>= 4: all)
+            const float s1 = in0 < 4 ? scale[row + 1] : s0;
             const unsigned w = c[i];
             float4_t o;
-            o.x = (float)((int)(w << 24) >> 24) * s;
-            o.y = (float)((int)(w << 16) >> 24) * s;
-            o.z = (float)((int)(w << 8) >> 24) * s;
-            o.w = (float)((int)w >> 24) * s;
+            o.x = (float)((int)(w << 24) >> 24) * s0;
+            o.y = (float)((int)(w << 16) >> 24) * (in0 > 1 ? s0 : s1);
+            o.z = (float)((int)(w << 8) >> 24) * (in0 > 2 ? s0 : s1);
+            o.w = (float)((int)w >> 24) * (in0 > 3 ? s0 : s1);
             __builtin_nontemporal_store(o, xv + idx);
         }
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (unsigned)(n & 3)) {
+        const int64_t i = (nv_total << 2) + threadIdx.x;
+        x[i] = (float)q[i] * scale[(n - 1) / cols];
     }
 }
 
@@ -460,8 +535,14 @@ int launch_quantize_rows(const float *x, int64_t rows, int64_t cols, int8_t *q, 
         VTL_Q_REG(1024, 4);
     else if (vec && cols <= 4 * 1024 * 16)
         VTL_Q_REG(1024, 16);
-    else if (vec)
+    else if (aligned(x, 16) && aligned(q, 4) && cols > 4 * 256 * 4)
         hipLaunchKernelGGL((quantize_rows_loop_kernel<1024, 4>), grid, dim3(1024), 0, st, x, cols, q,
+                           scale_out);
+    else if (aligned(x, 16) && aligned(q, 4) && cols >= 1024)
+        hipLaunchKernelGGL((quantize_rows_loop_kernel<256, 4>), grid, dim3(256), 0, st, x, cols, q,
+                           scale_out);
+    else if (aligned(x, 16) && aligned(q, 4) && cols >= 16)
+        hipLaunchKernelGGL((quantize_rows_loop_kernel<64, 4>), grid, dim3(64), 0, st, x, cols, q,
                            scale_out);
     else
         hipLaunchKernelGGL((quantize_rows_loop_kernel<256, 1>), grid, dim3(256), 0, st, x, cols, q,
@@ -485,7 +566,7 @@ int vtl_hip_absmax_f32(const float *x, int64_t rows, int64_t cols, int per_row, 
             return VTL_HIP_OK;
         if (cols == 0)
             return launch_fill_zero(absmax_out, rows, s);
-        const bool vec = (cols % 4 == 0) && aligned(x, 16);
+        const bool vec = aligned(x, 16);  // any row length: the kernel peels to the next 16-byte boundary
         if (vec && cols >= 8192)
             hipLaunchKernelGGL((absmax_rows_kernel<512, 4>), dim3((unsigned)rows), dim3(512), 0, s, x,
                                cols, absmax_out);
@@ -532,14 +613,15 @@ int vtl_hip_quantize_with_scale_f32_i8(const float *x, const float *scale, int64
     const int64_t row_len = per_row ? cols : rows * cols;
     const bool vec = aligned(x, 16) && aligned(q, 4) && (!per_row || cols % 4 == 0);
     const int64_t per_chunk = vec ? 4 * T * NV : T * NV;
-    if (per_row && vec && rows > 1 && cols < per_chunk) {
-        const int64_t nv_total = rows * (cols >> 2);
-        const int64_t nblocks = (nv_total + T * NV - 1) / (T * NV);
+    if (per_row && rows > 1 && cols >= 4 && cols < ((int64_t)1 << 31) - 4 * T * NV && aligned(x, 16) &&
+        aligned(q, 4) && (cols < 4 * T * NV || cols % 4 != 0)) {
+        const int64_t n = rows * cols;
+        const int64_t nblocks = ((n >> 2) + T * NV - 1) / (T * NV);
         if (nblocks > kMaxGridX)
             return VTL_HIP_ERR_UNSUPPORTED;
-        hipLaunchKernelGGL((quantize_scaled_short_rows_kernel<T, NV>), dim3((unsigned)nblocks), dim3(T), 0, s, x,
-                           scale, (unsigned)(cols >> 2), nv_total, q);
-        return check_launch("quantize_scaled_short_rows_kernel");
+        hipLaunchKernelGGL((quantize_scaled_flat_rows_kernel<T, NV>), dim3((unsigned)(nblocks > 0 ? nblocks : 1)),
+                           dim3(T), 0, s, x, scale, (unsigned)cols, n, q);
+        return check_launch("quantize_scaled_flat_rows_kernel");
     }
     const int64_t chunks = (row_len + per_chunk - 1) / per_chunk;
     const int64_t blocks = per_row ? rows * chunks : chunks;
@@ -599,14 +681,15 @@ int vtl_hip_dequantize_i8_f32(const int8_t *q, const float *scale, int64_t rows,
     const int64_t row_len = per_row ? cols : rows * cols;
     const bool vec = aligned(x, 16) && aligned(q, 4) && (!per_row || cols % 4 == 0);
     const int64_t per_chunk = vec ? 4 * T * NV : T * NV;
-    if (per_row && vec && rows > 1 && cols < per_chunk) {
-        const int64_t nv_total = rows * (cols >> 2);
-        const int64_t nblocks = (nv_total + T * NV - 1) / (T * NV);
+    if (per_row && rows > 1 && cols >= 4 && cols < ((int64_t)1 << 31) - 4 * T * NV && aligned(x, 16) &&
+        aligned(q, 4) && (cols < 4 * T * NV || cols % 4 != 0)) {
+        const int64_t n = rows * cols;
+        const int64_t nblocks = ((n >> 2) + T * NV - 1) / (T * NV);
         if (nblocks > kMaxGridX)
             return VTL_HIP_ERR_UNSUPPORTED;
-        hipLaunchKernelGGL((dequantize_short_rows_kernel<T, NV>), dim3((unsigned)nblocks), dim3(T), 0, s, q, scale,
-                           (unsigned)(cols >> 2), nv_total, x);
-        return check_launch("dequantize_short_rows_kernel");
+        hipLaunchKernelGGL((dequantize_flat_rows_kernel<T, NV>), dim3((unsigned)(nblocks > 0 ? nblocks : 1)),
+                           dim3(T), 0, s, q, scale, (unsigned)cols, n, x);
+        return check_launch("dequantize_flat_rows_kernel");
     }
     const int64_t chunks = (row_len + per_chunk - 1) / per_chunk;
     const int64_t blocks = per_row ? rows * chunks : chunks;
