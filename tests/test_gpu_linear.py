@@ -135,10 +135,13 @@ def test_session_reuses_buffers_on_second_forward(hip):
     layer.release()
 
 
-@pytest.mark.parametrize("nk", [(2048, 256), (2050, 512), (3001, 4096), (2077, 1280)])
+@pytest.mark.parametrize("nk", [(2048, 256), (2050, 512), (3001, 4096), (2077, 1280), (1, 16), (7, 48), (300, 784),
+                                (14336, 4080), (4097, 5120), (2048, 8192), (1000, 7168), (2050, 8208),
+                                (64, 11008)])
 def test_single_token_fused_decode_equals_two_launch_path(hip, nk, monkeypatch):
-    """M = 1 takes the kernel that quantizes the token itself; it must give the
-    bits of the quantize-then-linear path and of the oracle."""
+    """M = 1 takes the matrix-vector kernel that quantizes the token itself (rows of
+    up to 8192 codes, any multiple of 16; longer rows take two launches); it must
+    give the bits of the quantize-then-linear path and of the oracle."""
     n, k = nk
     rng = np.random.Generator(np.random.Philox(n + k))
     x = rng.standard_normal((1, k), dtype=np.float32)

@@ -692,214 +692,121 @@ __device__ __forceinline__ void lds_barrier()
     asm volatile("" ::: "memory");
 }
 
-// Decode with the activation quantization fused in, for M <= MR rows of f32
-// activations with K <= 4096 (used for a single token): every workgroup first computes the row scales itself
-// (absmax / 127 over the whole row - M x K floats from L2, cheap for a few rows)
-// and quantizes the rows into LDS, while its first weight chunks are already
-// in flight; then it streams its 32 weight rows exactly like
-// linear_skinny_kernel, reading the activation operand from that LDS copy.
-// The codes and scales are the ones quantize_rows_reg_kernel would produce
-// (same scale division, same quant_code), so results are bit-identical to the
-// two-launch path; one launch and its latency are saved.
-template <int NWAVE, int STAGES, int MR>
-__global__ __launch_bounds__(64 * NWAVE) void linear_skinny_dynquant_kernel(const GemmArgs g)
+// Single token (M = 1): a matrix-vector product bound by reading Wq once, done
+// without LDS staging and without MFMA.  With DYNQ the row arrives as f32 and
+// every workgroup quantizes it itself (K floats from L2, the arithmetic of the
+// row quantizer, codes exchanged through LDS) while the first weight rows of
+// its waves are already in flight; otherwise the codes and their scale are
+// read as given.  Each lane keeps its 16-byte pieces of the codes in registers
+// (KV of them, K <= 1024 * KV) for all rows.  A wave owns a run of consecutive
+// weight rows: a row is up to KV fully coalesced 1 KiB loads straight into
+// registers (cached loads: between launches the weights stay in the last-level
+// cache, non-temporal ones measured 20-40 % slower), two rows are in flight
+// while the current one goes through 4 * KV dot4 instructions and a
+// cross-lane sum.  Requires K % 16 == 0, the row and Wq 16-byte aligned.
+template <int KV, int NWAVE, bool DYNQ, bool F32OUT>
+__global__ __launch_bounds__(64 * NWAVE) void linear_gemv_kernel(const GemmArgs g)
 {
-    using namespace vtlhip::qdev;
-    constexpr int NT = 64 * NWAVE;
-    constexpr int BK = 256;
-    constexpr int SLOT = 32 * BK;  // 8 KiB of weights
-    constexpr int LOADS = 8;
-    constexpr int KS = BK / 32;
-    static_assert((STAGES - 1) * LOADS <= 63, "vmcnt is a 6-bit counter");
-    extern __shared__ __attribute__((aligned(16))) char smem[];
-    const int M = g.M, N = g.N, K = g.K;
-    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-    const int n0 = blockIdx.x * 32;
-    char *ring = smem + w * (STAGES * SLOT);
-    const int xstride = K + 16;  // bytes between activation rows in LDS (de-phases the banks)
-    char *xq = smem + NWAVE * STAGES * SLOT;                              // [MR][K + 16] codes
-    float *s_scale = reinterpret_cast<float *>(xq + MR * xstride);        // [MR]
-    float *s_red = s_scale + MR;                                          // [NWAVE][MR]
+    constexpr int T = 64 * NWAVE;
+    constexpr int XV = (256 * KV + T - 1) / T;  // float4 of x per thread
+    constexpr int DEPTH = 2, RING = DEPTH + 1;
+    __shared__ float red[NWAVE];
+    __shared__ __attribute__((aligned(16))) int8_t xq[DYNQ ? 1024 * KV : 16];
+    const int N = g.N, K = g.K;
+    const int kv = K >> 4;  // 16-byte pieces of a row
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int64_t waves = (int64_t)gridDim.x * NWAVE;
+    const int rows_per_wave = (int)((N + waves - 1) / waves);
+    const int64_t r0 = ((int64_t)blockIdx.x * NWAVE + w) * rows_per_wave;
+    const int64_t r1 = r0 + rows_per_wave < N ? r0 + rows_per_wave : N;
 
-    const int kc_all = K / BK;
-    const int kc_begin = (int)((int64_t)kc_all * w / NWAVE);
-    const int kc_end = (int)((int64_t)kc_all * (w + 1) / NWAVE);
-    const int KC = kc_end - kc_begin;
-
-    const int lrow = lane >> 4;
-    const int8_t *pw[LOADS];
+    v4i wb[RING][KV];
+    auto load_row = [&](int64_t r, v4i (&dst)[KV]) {
+        const v4i *p = reinterpret_cast<const v4i *>(g.Bt + r * K) + lane;
 #pragma unroll
-    for (int j = 0; j < LOADS; j++) {
-        const int row = lrow + 4 * j;
-        const int lc = (lane & 15) ^ (row & 15);
-        pw[j] = g.Bt + (int64_t)min(n0 + row, N - 1) * K + (int64_t)kc_begin * BK + lc * 16;
-    }
-    auto issue = [&](int c, int st) {
-        char *sw_ = ring + st * SLOT;
-        const int64_t ko = (int64_t)c * BK;
-#pragma unroll
-        for (int j = 0; j < LOADS; j++)
-            __builtin_amdgcn_global_load_lds(VTL_GPTR(pw[j] + ko), VTL_LPTR(sw_ + j * 1024), 16, 0, 0);
+        for (int j = 0; j < KV; j++)
+            dst[j] = (64 * j + lane < kv) ? p[64 * j] : v4i{0, 0, 0, 0};
     };
-    // ---- row scales and codes of the activations: each row is read once and kept in
-    //      registers between the absmax pass and the quantize pass (K <= 4 * NT * RC).
-    //      The activation loads are issued BEFORE the weight loads: vector-memory
-    //      results return in issue order, so the (cached) activations arrive first
-    //      and are quantized while the first weight chunks are still on their way ----
-    constexpr int RC = 8;
-    const int nv = K >> 2;
-    float4_t xr[MR][RC];
-    float mx[MR];
-    // The loads are written as instructions so that the wait below can name how
-    // many younger loads may stay in flight; the compiler's own bookkeeping would
-    // wait for the weight loads as well.  Lanes past the row re-read its last
-    // vector and discard it.
 #pragma unroll
-    for (int m = 0; m < MR; m++) {
-        const float4_t *xv = reinterpret_cast<const float4_t *>(g.xf32 + (int64_t)min(m, M - 1) * K);
-#pragma unroll
-        for (int r = 0; r < RC; r++) {
-            const int i = tid + r * NT;
-            const float4_t *src = xv + (i < nv ? i : nv - 1);
-            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(xr[m][r]) : "v"(src) : "memory");
-        }
-    }
-    int issued = 0;
-#pragma unroll
-    for (int st = 0; st < STAGES - 1; st++)
-        if (st < KC) {
-            issue(st, st);
-            issued += LOADS;
-        }
-    // activations have arrived once at most the weight loads issued after them are outstanding
-    if (issued == (STAGES - 1) * LOADS)
-        wait_vmcnt<(STAGES - 1) * LOADS>();
-    else
-        wait_vmcnt<0>();
-#pragma unroll
-    for (int m = 0; m < MR; m++)
-#pragma unroll
-        for (int r = 0; r < RC; r++) {
-            asm volatile("" : "+v"(xr[m][r]));   // uses stay below the wait
-            if (tid + r * NT >= nv)
-                xr[m][r] = float4_t{0.f, 0.f, 0.f, 0.f};
-        }
-#pragma unroll
-    for (int m = 0; m < MR; m++) {
-        float a = 0.0f;
-#pragma unroll
-        for (int r = 0; r < RC; r++)
-            a = absmax4(a, xr[m][r]);
-        mx[m] = wave_max(a);
-    }
-    if (lane == 0) {
-#pragma unroll
-        for (int m = 0; m < MR; m++)
-            s_red[w * MR + m] = mx[m];
-    }
-    lds_barrier();
-    if (tid < MR) {
-        float a = s_red[tid];
-        for (int ww = 1; ww < NWAVE; ww++)
-            a = fmaxf(a, s_red[ww * MR + tid]);
-        s_scale[tid] = a / 127.0f;
-    }
-    lds_barrier();
-#pragma unroll
-    for (int m = 0; m < MR; m++) {
-        const QuantScale p = make_quant_scale(s_scale[m]);
-        unsigned *dst = reinterpret_cast<unsigned *>(xq + m * xstride);
-#pragma unroll
-        for (int r = 0; r < RC; r++) {
-            const int i = tid + r * NT;
-            if (i < nv)
-                dst[i] = quant4(xr[m][r], p);
-        }
-    }
-    lds_barrier();
+    for (int d = 0; d < DEPTH; d++)
+        if (r0 + d < r1)
+            load_row(r0 + d, wb[d]);
 
-    v16i acc0, acc1;
+    v4i xc[KV];
+    float sx;
+    if constexpr (DYNQ) {
+        const f4 *xv = reinterpret_cast<const f4 *>(g.xf32);
+        f4 xr[XV];
+        float m = 0.0f;
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-        acc0[r] = 0;
-        acc1[r] = 0;
-    }
-    const int frow = lane & 31, fh = lane >> 5;
-    const int xrow = frow & (MR - 1);  // absent activation rows alias existing ones
-    int woff[KS];
-#pragma unroll
-    for (int s = 0; s < KS; s++)
-        woff[s] = frow * BK + ((((2 * s + fh) ^ frow) & 15) << 4);
-    const char *xbase = xq + xrow * xstride + kc_begin * BK + fh * 16;
-
-    int st_c = 0, st_l = STAGES - 1;
-    for (int c = 0; c < KC; c++) {
-        if (c + STAGES - 1 < KC) {
-            issue(c + STAGES - 1, st_l);
-            wait_vmcnt<(STAGES - 1) * LOADS>();
-        } else {
-            wait_vmcnt<0>();
+        for (int i = 0; i < XV; i++) {
+            const int idx = i * T + threadIdx.x;
+            xr[i] = idx < (K >> 2) ? xv[idx] : f4{0.f, 0.f, 0.f, 0.f};
+            m = vtlhip::qdev::absmax4(m, xr[i]);
         }
-        const char *sw_ = ring + st_c * SLOT;
-        const char *sx_ = xbase + c * BK;
-        v4i wf[KS], xf[KS];
+        m = vtlhip::qdev::wave_max(m);
+        if (lane == 0)
+            red[w] = m;
+        lds_barrier();
+        float am = red[0];
 #pragma unroll
-        for (int s = 0; s < KS; s++) {
-            wf[s] = *reinterpret_cast<const v4i *>(sw_ + woff[s]);
-            xf[s] = *reinterpret_cast<const v4i *>(sx_ + 32 * s);
-        }
+        for (int i = 1; i < NWAVE; i++)
+            am = fmaxf(am, red[i]);
+        sx = am / 127.0f;
+        const vtlhip::qdev::QuantScale qp = vtlhip::qdev::make_quant_scale(sx);
 #pragma unroll
-        for (int s = 0; s < KS; s += 2) {
-            acc0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[s], xf[s], acc0, 0, 0, 0);
-            acc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[s + 1], xf[s + 1], acc1, 0, 0, 0);
+        for (int i = 0; i < XV; i++) {
+            const int idx = i * T + threadIdx.x;
+            if (idx < 256 * KV)  // pieces past K are written as zeros
+                reinterpret_cast<unsigned *>(xq)[idx] = vtlhip::qdev::quant4(xr[i], qp);
         }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        st_c = (st_c + 1 == STAGES) ? 0 : st_c + 1;
-        st_l = (st_l + 1 == STAGES) ? 0 : st_l + 1;
+        lds_barrier();
+#pragma unroll
+        for (int j = 0; j < KV; j++)
+            xc[j] = reinterpret_cast<const v4i *>(xq)[64 * j + lane];
+    } else {
+        sx = F32OUT ? g.sa[0] : 0.0f;
+        const v4i *p = reinterpret_cast<const v4i *>(g.A) + lane;
+#pragma unroll
+        for (int j = 0; j < KV; j++)
+            xc[j] = (64 * j + lane < kv) ? p[64 * j] : v4i{0, 0, 0, 0};
     }
 
-    // ---- add the waves' partial tiles up through LDS: part[wave][m][n] (rings are free now) ----
-    __syncthreads();
-    int *part = reinterpret_cast<int *>(smem);
-    {
-        const int m = lane & 31, nb = (lane >> 5) * 4;
-        if (m < MR) {
+    for (int64_t rb = r0; rb < r1; rb += RING) {
 #pragma unroll
-            for (int rq = 0; rq < 4; rq++) {
-                v4i v;
+        for (int u = 0; u < RING; u++) {
+            const int64_t r = rb + u;
+            if (r >= r1)
+                break;
+            if (r + DEPTH < r1)
+                load_row(r + DEPTH, wb[(u + DEPTH) % RING]);
+            int acc = 0;
 #pragma unroll
-                for (int k = 0; k < 4; k++)
-                    v[k] = acc0[rq * 4 + k] + acc1[rq * 4 + k];
-                *reinterpret_cast<v4i *>(part + w * (MR * 32) + m * 32 + 8 * rq + nb) = v;
-            }
-        }
-    }
-    __syncthreads();
-    for (int item = tid; item < MR * 8; item += NT) {
-        const int m = item >> 3, nq = (item & 7) * 4;
-        v4i sum = *reinterpret_cast<const v4i *>(part + m * 32 + nq);
+            for (int j = 0; j < KV; j++)
 #pragma unroll
-        for (int ww = 1; ww < NWAVE; ww++)
-            sum += *reinterpret_cast<const v4i *>(part + ww * (MR * 32) + m * 32 + nq);
-        if (m >= M)
-            continue;
-        const int n = n0 + nq;
-        const float a = s_scale[m];
-        float *yrow = reinterpret_cast<float *>(g.out) + (int64_t)m * N;
+                for (int c = 0; c < 4; c++)
+                    acc = __builtin_amdgcn_sdot4(wb[u][j][c], xc[j][c], acc, false);
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            if (n + k < N) {
-                const float sc = a * g.sw[(int64_t)(n + k) * g.sw_stride];
-                float v = (float)sum[k] * sc;
-                if (g.bias)
-                    v = v + g.bias[n + k];
-                if (g.relu && v < 0.0f)
-                    v = 0.0f;
-                yrow[n + k] = v;
+            for (int off = 32; off > 0; off >>= 1)
+                acc += __shfl_xor(acc, off, 64);
+            if (lane == 0) {
+                if constexpr (F32OUT) {
+                    const float sc = sx * g.sw[r * g.sw_stride];
+                    float y = (float)acc * sc;
+                    if (g.bias)
+                        y = y + g.bias[r];
+                    if (g.relu && y < 0.0f)
+                        y = 0.0f;
+                    reinterpret_cast<float *>(g.out)[r] = y;
+                } else {
+                    reinterpret_cast<int32_t *>(g.out)[r] = acc;
+                }
             }
         }
     }
 }
+
+
 
 // Any shape, any alignment: one output per thread.  Only used when K is not a
 // multiple of 16 or a pointer is not 16-byte aligned.
@@ -1182,21 +1089,31 @@ int launch_skinny(const GemmArgs &g, hipStream_t st)
     return launch_skinny_cfg<2, 2, 4, F32OUT>(g, st);
 }
 
-template <int MR>
-int launch_skinny_dynquant(const GemmArgs &g, hipStream_t st)
+// Single-token linear (M = 1, K % 16 == 0, K <= 8192, operands 16-byte aligned).
+template <bool DYNQ, bool F32OUT>
+int launch_gemv(const GemmArgs &g, hipStream_t st)
 {
-    constexpr int NWAVE = 2, STAGES = 4;  // a deep ring: weights keep streaming while the rows are quantized
-    const int lds = NWAVE * STAGES * 8192 + MR * (g.K + 16) + (MR + NWAVE * MR) * (int)sizeof(float) + 16;
-    static PerDevice<int> attr_lds_dev;
-    int &attr_lds = attr_lds_dev.get();
-    auto kern = linear_skinny_dynquant_kernel<NWAVE, STAGES, MR>;
-    if (lds > attr_lds) {  // the LDS need grows with K
-        VTL_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-        attr_lds = lds;
+    constexpr int NWAVE = 4;
+    // about four workgroups per compute unit, a whole number of rows per wave
+    const int64_t waves_wanted = 4096;
+    const int rows_per_wave = (int)((g.N + waves_wanted - 1) / waves_wanted);
+    const int64_t waves = (g.N + rows_per_wave - 1) / rows_per_wave;
+    const dim3 grid((unsigned)((waves + NWAVE - 1) / NWAVE)), block(64 * NWAVE);
+    switch ((g.K + 1023) / 1024) {
+    case 1: hipLaunchKernelGGL((linear_gemv_kernel<1, NWAVE, DYNQ, F32OUT>), grid, block, 0, st, g); break;
+    case 2: hipLaunchKernelGGL((linear_gemv_kernel<2, NWAVE, DYNQ, F32OUT>), grid, block, 0, st, g); break;
+    case 3: hipLaunchKernelGGL((linear_gemv_kernel<3, NWAVE, DYNQ, F32OUT>), grid, block, 0, st, g); break;
+    case 4: hipLaunchKernelGGL((linear_gemv_kernel<4, NWAVE, DYNQ, F32OUT>), grid, block, 0, st, g); break;
+    case 5:
+    case 6: hipLaunchKernelGGL((linear_gemv_kernel<6, NWAVE, DYNQ, F32OUT>), grid, block, 0, st, g); break;
+    default: hipLaunchKernelGGL((linear_gemv_kernel<8, NWAVE, DYNQ, F32OUT>), grid, block, 0, st, g); break;
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)((g.N + 31) / 32)), dim3(64 * NWAVE), lds, st, g);
-    return check_launch("linear_skinny_dynquant_kernel");
+    return check_launch("linear_gemv_kernel");
+}
+
+inline bool gemv_applies(const void *row, const void *w, int K)
+{
+    return K % 16 == 0 && K <= 8192 && aligned16(row) && aligned16(w) && !getenv("VTL_HIP_NO_GEMV");
 }
 
 template <bool F32OUT>
@@ -1234,6 +1151,11 @@ int launch_gemm(const GemmArgs &g_in, hipStream_t st)
         g.Bt = ws + a_bytes;
         g.K = Kp;
     }
+    // one row: matrix-vector product (very short rows go to the small-product kernel; long rows
+    // of a tall matrix measured a few percent better in the MFMA weight-streaming kernel)
+    if (g.M == 1 && g.K >= 256 && (g.K <= 4096 || g.N < 8192) && gemv_applies(g.A, g.Bt, g.K) &&
+        !getenv("VTL_HIP_GEMM_CONFIG") && !getenv("VTL_HIP_GEMM_SMALL"))
+        return launch_gemv<false, F32OUT>(g, st);
     if (g.K % 256 == 0 && g.M <= 32 && g.N >= 2048 && !getenv("VTL_HIP_GEMM_CONFIG"))
         return launch_skinny<F32OUT>(g, st);  // weight streaming: enough row blocks to fill the chip
     const int64_t t32 = (int64_t)((g.M + 31) / 32) * ((g.N + 31) / 32);
@@ -1322,14 +1244,12 @@ int vtl_hip_linear_f32_dynquant(const float *X, const int8_t *Wq, const float *s
     if (workspace && (workspace_bytes < vtl_hip_linear_f32_dynquant_workspace(M, K) ||
                       (reinterpret_cast<uintptr_t>(workspace) & 15)))
         return VTL_HIP_ERR_INVALID_ARG;
-    if (M == 1 && K % 256 == 0 && K <= 4096 && N >= 2048 && aligned16(X) && aligned16(Wq) &&
-        !getenv("VTL_HIP_NO_FUSED_DECODE")) {
-        // a single token: quantize it inside the weight-streaming kernel (one launch instead of
-        // two; measured 15 % faster at N = 14336, K = 4096; for two rows 13.5 us against 12.8 us
-        // for the two launches, and from three rows on the registers no longer hold the rows).  The
-        // workspace stays unused.  VTL_HIP_NO_FUSED_DECODE forces the two-launch path (tests).
+    if (M == 1 && gemv_applies(X, Wq, K) && !getenv("VTL_HIP_NO_FUSED_DECODE")) {
+        // a single token: quantized inside the matrix-vector kernel, one launch instead of two
+        // (N = 14336, K = 4096: 9.5 us against 12.8 us).  The workspace stays unused.
+        // VTL_HIP_NO_FUSED_DECODE forces the two-launch path (tests).
         GemmArgs g{nullptr, Wq, Y, nullptr, sw, bias, M, N, K, 1, 1, relu ? 1 : 0, 1, nullptr, X};
-        return launch_skinny_dynquant<1>(g, current_stream());
+        return launch_gemv<true, true>(g, current_stream());
     }
     if (!workspace) {   // no caller scratch: stage in the library's own buffer
         workspace = vtlhip::library_workspace(vtl_hip_linear_f32_dynquant_workspace(M, K), 1);
