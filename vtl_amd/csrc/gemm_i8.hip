@@ -715,10 +715,10 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_gemv_kernel(const GemmArgs 
     const int N = g.N, K = g.K;
     const int kv = K >> 4;  // 16-byte pieces of a row
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    const int64_t waves = (int64_t)gridDim.x * NWAVE;
-    const int rows_per_wave = (int)((N + waves - 1) / waves);
-    const int64_t r0 = ((int64_t)blockIdx.x * NWAVE + w) * rows_per_wave;
-    const int64_t r1 = r0 + rows_per_wave < N ? r0 + rows_per_wave : N;
+    // rows are dealt out cyclically: wave i of W takes rows i, i + W, i + 2 W, ... so that at any
+    // moment the waves of the chip read one contiguous stretch of the matrix
+    const int64_t W = (int64_t)gridDim.x * NWAVE;
+    const int64_t r0 = (int64_t)blockIdx.x * NWAVE + w, r1 = N;
 
     v4i wb[RING][KV];
     auto load_row = [&](int64_t r, v4i (&dst)[KV]) {
@@ -729,8 +729,8 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_gemv_kernel(const GemmArgs 
     };
 #pragma unroll
     for (int d = 0; d < DEPTH; d++)
-        if (r0 + d < r1)
-            load_row(r0 + d, wb[d]);
+        if (r0 + d * W < r1)
+            load_row(r0 + d * W, wb[d]);
 
     v4i xc[KV];
     float sx;
@@ -772,14 +772,25 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_gemv_kernel(const GemmArgs 
             xc[j] = (64 * j + lane < kv) ? p[64 * j] : v4i{0, 0, 0, 0};
     }
 
-    for (int64_t rb = r0; rb < r1; rb += RING) {
+    // lane u of the wave looks after its u-th row: scale and bias are fetched now, the sum is
+    // parked in the lane when the row is done, the epilogue runs once after the loop
+    const int64_t my_row = r0 + (int64_t)lane * W;
+    const bool mine = my_row < r1;
+    float swv = 0.0f, bv = 0.0f;
+    if (F32OUT && mine) {
+        swv = g.sw[my_row * g.sw_stride];
+        if (g.bias)
+            bv = g.bias[my_row];
+    }
+    int res = 0, it = 0;
+    for (int64_t rb = r0; rb < r1; rb += RING * W) {
 #pragma unroll
         for (int u = 0; u < RING; u++) {
-            const int64_t r = rb + u;
+            const int64_t r = rb + u * W;
             if (r >= r1)
                 break;
-            if (r + DEPTH < r1)
-                load_row(r + DEPTH, wb[(u + DEPTH) % RING]);
+            if (r + DEPTH * W < r1)
+                load_row(r + DEPTH * W, wb[(u + DEPTH) % RING]);
             int acc = 0;
 #pragma unroll
             for (int j = 0; j < KV; j++)
@@ -789,19 +800,21 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_gemv_kernel(const GemmArgs 
 #pragma unroll
             for (int off = 32; off > 0; off >>= 1)
                 acc += __shfl_xor(acc, off, 64);
-            if (lane == 0) {
-                if constexpr (F32OUT) {
-                    const float sc = sx * g.sw[r * g.sw_stride];
-                    float y = (float)acc * sc;
-                    if (g.bias)
-                        y = y + g.bias[r];
-                    if (g.relu && y < 0.0f)
-                        y = 0.0f;
-                    reinterpret_cast<float *>(g.out)[r] = y;
-                } else {
-                    reinterpret_cast<int32_t *>(g.out)[r] = acc;
-                }
-            }
+            res = (lane == it) ? acc : res;
+            it++;
+        }
+    }
+    if (mine) {
+        if constexpr (F32OUT) {
+            const float sc = sx * swv;
+            float y = (float)res * sc;
+            if (g.bias)
+                y = y + bv;
+            if (g.relu && y < 0.0f)
+                y = 0.0f;
+            reinterpret_cast<float *>(g.out)[my_row] = y;
+        } else {
+            reinterpret_cast<int32_t *>(g.out)[my_row] = res;
         }
     }
 }
@@ -1093,10 +1106,9 @@ int launch_skinny(const GemmArgs &g, hipStream_t st)
 template <bool DYNQ, bool F32OUT>
 int launch_gemv(const GemmArgs &g, hipStream_t st)
 {
-    constexpr int NWAVE = 4;
-    // about four workgroups per compute unit, a whole number of rows per wave
-    const int64_t waves_wanted = 4096;
-    const int rows_per_wave = (int)((g.N + waves_wanted - 1) / waves_wanted);
+    constexpr int NWAVE = 8;
+    // about sixteen waves per compute unit, and every wave the same number of rows
+    const int rows_per_wave = (g.N + 4095) / 4096;
     const int64_t waves = (g.N + rows_per_wave - 1) / rows_per_wave;
     const dim3 grid((unsigned)((waves + NWAVE - 1) / NWAVE)), block(64 * NWAVE);
     switch ((g.K + 1023) / 1024) {
@@ -1111,9 +1123,10 @@ int launch_gemv(const GemmArgs &g, hipStream_t st)
     return check_launch("linear_gemv_kernel");
 }
 
-inline bool gemv_applies(const void *row, const void *w, int K)
+// N <= 64 * 4096: a wave parks one sum per lane.
+inline bool gemv_applies(const void *row, const void *w, int N, int K)
 {
-    return K % 16 == 0 && K <= 8192 && aligned16(row) && aligned16(w) && !getenv("VTL_HIP_NO_GEMV");
+    return K % 16 == 0 && K <= 8192 && N <= 64 * 4096 && aligned16(row) && aligned16(w) && !getenv("VTL_HIP_NO_GEMV");
 }
 
 template <bool F32OUT>
@@ -1153,7 +1166,7 @@ int launch_gemm(const GemmArgs &g_in, hipStream_t st)
     }
     // one row: matrix-vector product (very short rows go to the small-product kernel; long rows
     // of a tall matrix measured a few percent better in the MFMA weight-streaming kernel)
-    if (g.M == 1 && g.K >= 256 && (g.K <= 4096 || g.N < 8192) && gemv_applies(g.A, g.Bt, g.K) &&
+    if (g.M == 1 && g.K >= 256 && (g.K <= 4096 || g.N < 8192) && gemv_applies(g.A, g.Bt, g.N, g.K) &&
         !getenv("VTL_HIP_GEMM_CONFIG") && !getenv("VTL_HIP_GEMM_SMALL"))
         return launch_gemv<false, F32OUT>(g, st);
     if (g.K % 256 == 0 && g.M <= 32 && g.N >= 2048 && !getenv("VTL_HIP_GEMM_CONFIG"))
@@ -1244,7 +1257,7 @@ int vtl_hip_linear_f32_dynquant(const float *X, const int8_t *Wq, const float *s
     if (workspace && (workspace_bytes < vtl_hip_linear_f32_dynquant_workspace(M, K) ||
                       (reinterpret_cast<uintptr_t>(workspace) & 15)))
         return VTL_HIP_ERR_INVALID_ARG;
-    if (M == 1 && gemv_applies(X, Wq, K) && !getenv("VTL_HIP_NO_FUSED_DECODE")) {
+    if (M == 1 && gemv_applies(X, Wq, N, K) && !getenv("VTL_HIP_NO_FUSED_DECODE")) {
         // a single token: quantized inside the matrix-vector kernel, one launch instead of two
         // (N = 14336, K = 4096: 9.5 us against 12.8 us).  The workspace stays unused.
         // VTL_HIP_NO_FUSED_DECODE forces the two-launch path (tests).
