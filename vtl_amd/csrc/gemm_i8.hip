@@ -692,6 +692,21 @@ __device__ __forceinline__ void lds_barrier()
     asm volatile("" ::: "memory");
 }
 
+// Sum of an int over the 64 lanes of a wave, the same value returned to every
+// lane: cross-lane moves inside the VALU (DPP) instead of six trips through the
+// LDS crossbar.  Quads, half rows and rows by mirroring, then lane 15 of each
+// row into the next row and lane 31 into the upper half; lane 63 holds the sum.
+__device__ __forceinline__ int wave_sum_i32(int v)
+{
+    v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, false);   // quad_perm [1,0,3,2]
+    v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, false);   // quad_perm [2,3,0,1]
+    v += __builtin_amdgcn_update_dpp(0, v, 0x141, 0xF, 0xF, false);  // row_half_mirror
+    v += __builtin_amdgcn_update_dpp(0, v, 0x140, 0xF, 0xF, false);  // row_mirror
+    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xA, 0xF, false);  // row_bcast:15 into rows 1 and 3
+    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xC, 0xF, false);  // row_bcast:31 into rows 2 and 3
+    return __builtin_amdgcn_readlane(v, 63);
+}
+
 // Single token (M = 1): a matrix-vector product bound by reading Wq once, done
 // without LDS staging and without MFMA.  With DYNQ the row arrives as f32 and
 // every workgroup quantizes it itself (K floats from L2, the arithmetic of the
@@ -797,9 +812,7 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_gemv_kernel(const GemmArgs 
 #pragma unroll
                 for (int c = 0; c < 4; c++)
                     acc = __builtin_amdgcn_sdot4(wb[u][j][c], xc[j][c], acc, false);
-#pragma unroll
-            for (int off = 32; off > 0; off >>= 1)
-                acc += __shfl_xor(acc, off, 64);
+            acc = wave_sum_i32(acc);
             res = (lane == it) ? acc : res;
             it++;
         }
