@@ -12,12 +12,27 @@ namespace qdev {
 typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef int int4_t __attribute__((ext_vector_type(4)));
 
+// Max over the 64 lanes of a wave, returned to every lane: cross-lane moves
+// inside the VALU (DPP) - quads, half rows and rows by mirroring, then lane 15
+// of each row into the next row and lane 31 into the upper half; lane 63 holds
+// the result.  Lanes a move does not reach see 0, the identity for the
+// non-negative values this is used on.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_max_step(float v)
+{
+    const int t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xF, false);
+    return fmaxf(v, __int_as_float(t));
+}
+
 __device__ __forceinline__ float wave_max(float v)
 {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1)
-        v = fmaxf(v, __shfl_xor(v, off, 64));
-    return v;
+    v = dpp_max_step<0xB1, 0xF>(v);   // quad_perm [1,0,3,2]
+    v = dpp_max_step<0x4E, 0xF>(v);   // quad_perm [2,3,0,1]
+    v = dpp_max_step<0x141, 0xF>(v);  // row_half_mirror
+    v = dpp_max_step<0x140, 0xF>(v);  // row_mirror
+    v = dpp_max_step<0x142, 0xA>(v);  // row_bcast:15 into rows 1 and 3
+    v = dpp_max_step<0x143, 0xC>(v);  // row_bcast:31 into rows 2 and 3
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
 // Max over the workgroup; every thread gets the result.  smem holds T/64
