@@ -150,7 +150,7 @@ def bench_quant(timer: Timer, steps: int, warmup: int, cpu: bool):
     def d_step():
         capi.call("vtl_hip_dequantize_i8_f32", Q.ptr, S.ptr, rows, cols, 1, D.ptr)
 
-    for name, fn, kern in (("quantize", q_step, "quantize_rows_reg_kernel<1024,4>"),
+    for name, fn, kern in (("quantize", q_step, "quantize_rows_reg_kernel<1024,4,true>"),
                            ("dequantize", d_step, "dequantize_kernel<512,2,4>")):
         for _ in range(warmup):
             fn()

@@ -122,8 +122,11 @@ __global__ void scale_from_absmax_kernel(float *inout, int64_t n)
 
 // One workgroup per row; the row stays in registers between the absmax pass
 // and the quantize pass, so HBM sees 4 bytes in and 1 byte out per element.
-// Requires cols % 4 == 0 and cols <= 4 * T * NV.
-template <int T, int NV>
+// Requires cols % 4 == 0 and cols <= 4 * T * NV.  NT: non-temporal loads and
+// stores, for tensors far larger than the caches (16384^2: 209 us against 243 us
+// with cached accesses); small tensors that the next kernel reads back are
+// better left in the caches (the three-layer chain: 66 us against 69 us).
+template <int T, int NV, bool NT>
 __global__ __launch_bounds__(T) void quantize_rows_reg_kernel(const float *__restrict__ x,
                                                               int64_t cols, int8_t *__restrict__ q,
                                                               float *__restrict__ scale_out)
@@ -139,7 +142,7 @@ __global__ __launch_bounds__(T) void quantize_rows_reg_kernel(const float *__res
     for (int i = 0; i < NV; i++) {
         const int idx = i * T + threadIdx.x;
         if (idx < nv)
-            v[i] = __builtin_nontemporal_load(xv + idx);
+            v[i] = NT ? __builtin_nontemporal_load(xv + idx) : xv[idx];
         else
             v[i] = float4_t{0.f, 0.f, 0.f, 0.f};
     }
@@ -156,8 +159,12 @@ __global__ __launch_bounds__(T) void quantize_rows_reg_kernel(const float *__res
 #pragma unroll
     for (int i = 0; i < NV; i++) {
         const int idx = i * T + threadIdx.x;
-        if (idx < nv)
-            __builtin_nontemporal_store(quant4(v[i], p), qv + idx);
+        if (idx < nv) {
+            if (NT)
+                __builtin_nontemporal_store(quant4(v[i], p), qv + idx);
+            else
+                qv[idx] = quant4(v[i], p);
+        }
     }
 }
 
@@ -512,9 +519,16 @@ int launch_quantize_rows(const float *x, int64_t rows, int64_t cols, int8_t *q, 
         return launch_fill_zero(scale_out, rows, st);
     const bool vec = (cols % 4 == 0) && aligned(x, 16) && aligned(q, 4);
     const dim3 grid((unsigned)rows);
-#define VTL_Q_REG(T, NV)                                                                    \
-    hipLaunchKernelGGL((quantize_rows_reg_kernel<T, NV>), grid, dim3(T), 0, st, x, cols, q, \
-                       scale_out)
+    const bool nt = rows * cols > ((int64_t)16 << 20);  // more than 64 MiB of f32
+#define VTL_Q_REG(T, NV)                                                                               \
+    do {                                                                                               \
+        if (nt)                                                                                        \
+            hipLaunchKernelGGL((quantize_rows_reg_kernel<T, NV, true>), grid, dim3(T), 0, st, x, cols, q, \
+                               scale_out);                                                             \
+        else                                                                                           \
+            hipLaunchKernelGGL((quantize_rows_reg_kernel<T, NV, false>), grid, dim3(T), 0, st, x, cols, q, \
+                               scale_out);                                                             \
+    } while (0)
     // Workgroup sizes measured best per row length: one wave while the row
     // fits a wave's registers (no LDS, no barrier), 256 threads up to 4096
     // columns, 512 up to 8192, 1024 beyond (e.g. 65536 rows of 4096: 303 us
