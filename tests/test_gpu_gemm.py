@@ -169,6 +169,8 @@ def test_square_gemm_config_full_size(hip):
 # (few output tiles, long K) with uneven K ranges, and the register-staged
 # tile kernel (K % 128 != 0).
 ROUTED_SHAPES = [(1, 2048, 256), (1, 5, 256), (1, 4099, 4080), (1, 9000, 5120), (1, 300, 8192), (1, 2048, 8448),
+                 (1, 262200, 256),      # more rows than the matrix-vector kernel deals out
+
                  (3, 2050, 256), (8, 2048, 4096), (9, 2048, 768), (16, 2047, 1280),
                  (17, 2077, 1280), (32, 4096, 512), (31, 14336, 256), (5, 3001, 4096),
                  (256, 1024, 4096), (256, 512, 11008), (64, 128, 11008), (128, 256, 8192), (40, 200, 5504),
