@@ -112,7 +112,9 @@ int vtl_hip_dequantize_i8_f32(const int8_t *q, const float *scale, int64_t rows,
 /* C[M,N] (i32) = A[M,K] (i8) . Bt[N,K]^T (i8), exact.  The int8 counterpart
  * of la.matmul (la/la.v:38-55) / gate_matmul (autograd/gates_blas.v:6-23) /
  * gemm_cuda (tensor_cuda_d_cuda.v:155-177) with the second operand given
- * K-contiguous.  K <= 131072 so that |acc| <= K * 127^2 < 2^31. */
+ * K-contiguous.  K <= 131072 so that |acc| <= K * 127^2 < 2^31.  Any K and any
+ * alignment; K % 16 == 0 with A and Bt 16-byte aligned spares a repacking pass
+ * through scratch memory that the library allocates. */
 int vtl_hip_gemm_i8_i32(const int8_t *A, const int8_t *Bt, int32_t *C, int M, int N, int K);
 
 /* Y[m,n] = fl(fl(f32(acc) * fl(sa[m] * sw[n])) + bias[n]), ReLU if relu != 0
