@@ -367,7 +367,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=300)
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["all", "linear", "quant", "copy", "full"], default="all")
+    ap.add_argument("--only", choices=["all", "linear", "quant", "copy", "full", "other"], default="all")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 "
@@ -385,6 +385,9 @@ def main() -> int:
         return 0
     if args.only == "full":
         print(json.dumps({"full_precision": bench_full_precision(timer, args.steps, args.warmup)}))
+        return 0
+    if args.only == "other":
+        print(json.dumps({"other_configs": bench_other_configs(timer, args.steps, args.warmup)}))
         return 0
 
     lin = bench_linear(timer, args.steps, args.warmup, cpu) if args.only in ("all", "linear") else None

@@ -71,14 +71,14 @@ __device__ __forceinline__ void wait_vmcnt()
 }
 
 // Workgroups are dealt round-robin to the 8 XCDs; renumber them so that each
-// XCD (own L2) works on a compact patch of the tile grid, then walk the grid
-// in groups of 8 tile rows.
+// XCD (own L2) works on a compact patch of the tile grid (XCD x holds
+// total/8 tiles, one more when x < total%8), then walk the grid in groups of
+// 8 tile rows.
 __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int block, int &tile_m, int &tile_n)
 {
     const int total = tiles_m * tiles_n;
-    int pid = block;
-    if ((total & 7) == 0)
-        pid = (pid & 7) * (total >> 3) + (pid >> 3);
+    const int xcd = block & 7, rest = total & 7;
+    const int pid = xcd * (total >> 3) + min(xcd, rest) + (block >> 3);
     constexpr int GM = 8;
     const int group_size = GM * tiles_n;
     const int first_m = (pid / group_size) * GM;
