@@ -220,6 +220,41 @@ def test_every_kernel_family_matches_oracle(hip, mnk):
         h.release()
 
 
+# few-token kernel (2 <= M <= 8 rows of codes held in registers): every row count, every
+# row-length class (K <= 1024, 2048, 4096, 8192), K % 16 == 0 only, ragged N, more weight rows
+# than one batch of parked sums per wave (at K = 256 there are 8192 waves, a batch is 64 / MR
+# weight rows per wave: the last two shapes need two and three batches)
+FEW_TOKEN_SHAPES = [(2, 2048, 256), (2, 3001, 1008), (2, 2050, 2048), (2, 2048, 4096), (2, 2049, 8192),
+                    (3, 2048, 1024), (4, 4099, 1040), (4, 2048, 4096), (3, 2051, 8192), (4, 2048, 5120),
+                    (5, 2048, 512), (8, 2050, 2032), (7, 2048, 4096), (6, 5000, 3088), (8, 40000, 256),
+                    (2, 140000, 272), (4, 70001, 256), (8, 70001, 256), (5, 140000, 256)]
+
+
+@pytest.mark.parametrize("rows_kernel", ["1", "0", None])
+@pytest.mark.parametrize("mnk", FEW_TOKEN_SHAPES)
+def test_few_token_kernel_and_its_alternatives(hip, mnk, rows_kernel, monkeypatch):
+    """VTL_HIP_GEMV_ROWS=1 forces the few-token kernel wherever it applies, 0 keeps it
+    off, unset is the library's own choice: int32 sums and f32 epilogue are those of the oracle."""
+    if rows_kernel is None:
+        monkeypatch.delenv("VTL_HIP_GEMV_ROWS", raising=False)
+    else:
+        monkeypatch.setenv("VTL_HIP_GEMV_ROWS", rows_kernel)
+    m, n, k = mnk
+    a, bt, sa, sb, bias = workloads.square_int8_gemm(m, n, k, seed=m * 31 + n * 3 + k)
+    ref = oracle.gemm_i8_i32(a, bt, threads=CPU_THREADS)
+    assert np.array_equal(_gemm(a, bt), ref)
+    A, B, dsa, dsb, dbias = dev(a), dev(bt), dev(sa), dev(sb), dev(bias)
+    for relu, b_dev, b_host in ((True, dbias, bias), (False, None, None)):
+        y = linear_i8_hip(A, dsa, B, dsb, b_dev, relu=relu)
+        assert np.array_equal(y.cpu(), oracle.epilogue(ref, sa, sb, b_host, relu=relu))
+        y.release()
+    # one scale for all rows of A and one for all of W
+    y = linear_i8_hip(A, dev(sa[:1]), B, dev(sb[:1]), dbias, relu=False)
+    assert np.array_equal(y.cpu(), oracle.epilogue(ref, sa[:1], sb[:1], bias))
+    for h in (A, B, dsa, dsb, dbias, y):
+        h.release()
+
+
 @pytest.mark.parametrize("k", [2432, 2448, 80])   # 19 K steps of 128; the same plus a 16-byte tail; one partial step
 def test_forced_split_k_is_exact(hip, monkeypatch, k):
     """Every tile configuration with 1, 2, 3 and 8 K ranges gives the same int32 result

@@ -135,6 +135,48 @@ def test_session_reuses_buffers_on_second_forward(hip):
     layer.release()
 
 
+@pytest.mark.parametrize("mnk", [(2, 2048, 256), (2, 3001, 1008), (2, 2050, 2048), (2, 2048, 4096), (2, 2064, 3088),
+                                 (3, 2048, 1024), (4, 4099, 1040), (4, 2048, 2048), (3, 2051, 272),
+                                 (5, 2048, 512), (8, 2050, 1024), (7, 9000, 1008), (6, 2048, 16 * 17),
+                                 (8, 70001, 256)])
+def test_few_token_fused_decode_equals_two_launch_path(hip, mnk, monkeypatch):
+    """2 to 8 tokens with short rows take the few-token kernel whose workgroups quantize the
+    rows themselves (forced here for every size it is built for); it must give the bits of
+    the quantize-then-linear path and of the oracle, special values included."""
+    m, n, k = mnk
+    rng = np.random.Generator(np.random.Philox(m * 7 + n + k))
+    x = rng.standard_normal((m, k), dtype=np.float32)
+    x[0, :4] = [0.5, 1.5, -2.5, 3.5]
+    x[m - 1] *= np.float32(1e-30)            # a row with a tiny scale
+    if m > 2:
+        x[1] = 0.0                           # an all-zero row: scale 0, codes 0
+    w = rng.integers(-127, 128, (n, k), dtype=np.int8)
+    sw = (rng.uniform(0.5, 1.5, n) * 1e-3).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    X, W, SW, B = dev(x), dev(w), dev(sw), dev(bias)
+    want = oracle.linear_f32_dynquant(x, w, sw, bias, relu=True, threads=CPU_THREADS)
+    monkeypatch.setenv("VTL_HIP_GEMV_ROWS", "1")
+    fused = linear_f32_dynquant_hip(X, W, SW, B, relu=True).cpu()
+    monkeypatch.setenv("VTL_HIP_NO_FUSED_DECODE", "1")
+    plain = linear_f32_dynquant_hip(X, W, SW, B, relu=True).cpu()
+    monkeypatch.delenv("VTL_HIP_NO_FUSED_DECODE")
+    monkeypatch.delenv("VTL_HIP_GEMV_ROWS")
+    auto = linear_f32_dynquant_hip(X, W, SW, B, relu=True).cpu()
+    assert np.array_equal(fused, want) and np.array_equal(plain, want) and np.array_equal(auto, want)
+    monkeypatch.setenv("VTL_HIP_GEMV_ROWS", "1")
+    for special in (np.nan, np.inf, -np.inf):
+        xs = x.copy()
+        xs[0, 7] = special
+        xs[m - 1, k - 1] = special
+        S = dev(xs)
+        got = linear_f32_dynquant_hip(S, W, SW, None, relu=False).cpu()
+        ref = oracle.linear_f32_dynquant(xs, w, sw, None)
+        assert np.array_equal(got, ref, equal_nan=True), special
+        S.release()
+    for h in (X, W, SW, B):
+        h.release()
+
+
 @pytest.mark.parametrize("nk", [(2048, 256), (2050, 512), (3001, 4096), (2077, 1280), (1, 16), (7, 48), (300, 784),
                                 (14336, 4080), (4097, 5120), (2048, 8192), (1000, 7168), (2050, 8208),
                                 (64, 11008)])

@@ -756,6 +756,16 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_gemv_kernel(const GemmArgs 
     const int64_t W = (int64_t)gridDim.x * NWAVE;
     const int64_t r0 = (int64_t)blockIdx.x * NWAVE + w, r1 = N;
 
+    // the activations are asked for first: behind the weight rows they would wait for all of them
+    f4 xr[XV];
+    if constexpr (DYNQ) {
+        const f4 *xv = reinterpret_cast<const f4 *>(g.xf32);
+#pragma unroll
+        for (int i = 0; i < XV; i++) {
+            const int idx = i * T + threadIdx.x;
+            xr[i] = idx < (K >> 2) ? xv[idx] : f4{0.f, 0.f, 0.f, 0.f};
+        }
+    }
     v4i wb[RING][KV];
     auto load_row = [&](int64_t r, v4i (&dst)[KV]) {
         const v4i *p = reinterpret_cast<const v4i *>(g.Bt + r * K) + lane;
@@ -771,15 +781,10 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_gemv_kernel(const GemmArgs 
     v4i xc[KV];
     float sx;
     if constexpr (DYNQ) {
-        const f4 *xv = reinterpret_cast<const f4 *>(g.xf32);
-        f4 xr[XV];
         float m = 0.0f;
 #pragma unroll
-        for (int i = 0; i < XV; i++) {
-            const int idx = i * T + threadIdx.x;
-            xr[i] = idx < (K >> 2) ? xv[idx] : f4{0.f, 0.f, 0.f, 0.f};
+        for (int i = 0; i < XV; i++)
             m = vtlhip::qdev::absmax4(m, xr[i]);
-        }
         m = vtlhip::qdev::wave_max(m);
         if (lane == 0)
             red[w] = m;
@@ -853,6 +858,224 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_gemv_kernel(const GemmArgs 
     }
 }
 
+
+template <int CTRL>
+__device__ __forceinline__ int dpp_move(int v)
+{
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, false);
+}
+
+// MR per-lane partial sums (one per activation row) of the 64 lanes, added up
+// so that lane l ends with the wave's total for row l % MR.  Each folding step
+// halves the number of values a lane carries: the lanes of a pair keep one half
+// each and hand the other half over, so 8 rows cost 4 + 2 + 1 exchanges and
+// one more per remaining lane bit, instead of six per row.
+template <int MR>
+__device__ __forceinline__ int fold_rows(int (&a)[MR], int lane)
+{
+    if constexpr (MR == 1) {
+        return a[0];
+    } else {
+        constexpr int H = MR / 2;
+        const bool hi = (lane & H) != 0;
+        int b[H];
+#pragma unroll
+        for (int i = 0; i < H; i++) {
+            const int send = hi ? a[i] : a[i + H], keep = hi ? a[i + H] : a[i];
+            if constexpr (MR == 8)
+                b[i] = keep + dpp_move<0x141>(send);  // row_half_mirror: lane l of 8 <-> 7 - l
+            else if constexpr (MR == 4)
+                b[i] = keep + dpp_move<0x4E>(send);   // quad_perm [2,3,0,1]
+            else
+                b[i] = keep + dpp_move<0xB1>(send);   // quad_perm [1,0,3,2]
+        }
+        return fold_rows<H>(b, lane);
+    }
+}
+
+template <int MR>
+__device__ __forceinline__ int wave_sum_rows(int (&a)[MR], int lane)
+{
+    int v = fold_rows<MR>(a, lane);
+    if constexpr (MR < 4)
+        v += dpp_move<0x4E>(v);   // lanes l and l ^ 2
+    if constexpr (MR < 8)
+        v += dpp_move<0x124>(v);  // row_ror:4
+    v += dpp_move<0x128>(v);      // row_ror:8
+    // rows of 16 lanes: odd rows against even rows, then the upper half against the lower one
+    const auto r16 = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+    v = r16[0] + r16[1];
+    const auto r32 = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+    return r32[0] + r32[1];
+}
+
+// A few tokens (2 <= M <= MR, MR = 2, 4 or 8): the single-token kernel with MR
+// rows of codes in registers (16 * KV * MR bytes per lane), so every weight
+// row, loaded once and straight into registers, meets all of them: 4 * KV * MR
+// dot4 instructions and one folded cross-lane sum per weight row.  With DYNQ
+// every workgroup quantizes the MR activation rows itself, all threads sharing
+// the work (the arithmetic of the row quantizer), and the codes are exchanged
+// through LDS.  Sums are parked
+// 64 / MR weight rows at a time (lane l: row l % MR, weight row l / MR of the
+// batch) and then scaled and stored.  Requires K % 16 == 0, K <= 1024 * KV,
+// operands 16-byte aligned.
+template <int KV, int MR, int DEPTH, bool DYNQ, bool F32OUT>
+__global__ __launch_bounds__(512) void linear_gemv_rows_kernel(const GemmArgs g)
+{
+    constexpr int NWAVE = 8;
+    constexpr int RING = DEPTH + 1;
+    constexpr int SLOTS = 64 / MR;
+    __shared__ float s_sa[MR], s_rinv[MR];
+    __shared__ unsigned s_amax[MR];
+    __shared__ int s_fast[MR];
+    __shared__ __attribute__((aligned(16))) int8_t xq[DYNQ ? MR * 1024 * KV : 16];
+    const int M = g.M, N = g.N, K = g.K;
+    const int kv = K >> 4;  // 16-byte pieces of a row
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int64_t W = (int64_t)gridDim.x * NWAVE;
+    const int64_t r0 = (int64_t)blockIdx.x * NWAVE + w, r1 = N;
+
+    // The activations are asked for first: behind the weight rows they would wait for all of them.
+    // The MR rows are one flat run of 256 * KV * MR float4 pieces dealt out to the 512 threads, so
+    // the 64 pieces of a wave instruction belong to one row.
+    constexpr int PIECES = 256 * KV;                      // float4 per (padded) row
+    constexpr int XV = DYNQ ? (MR * PIECES) / 512 : 1;    // pieces per thread
+    static_assert(!DYNQ || (MR * PIECES) % 512 == 0, "whole pieces per thread");
+    f4 xr[XV];
+    if constexpr (DYNQ) {
+#pragma unroll
+        for (int i = 0; i < XV; i++) {
+            const int f = i * 512 + (int)threadIdx.x, row = f / PIECES, col = f % PIECES;
+            xr[i] = (row < M && col < (K >> 2))
+                        ? reinterpret_cast<const f4 *>(g.xf32 + (int64_t)row * K)[col]
+                        : f4{0.f, 0.f, 0.f, 0.f};
+        }
+    }
+    v4i wb[RING][KV];
+    auto load_row = [&](int64_t r, v4i (&dst)[KV]) {
+        const v4i *p = reinterpret_cast<const v4i *>(g.Bt + r * K) + lane;
+#pragma unroll
+        for (int j = 0; j < KV; j++)
+            dst[j] = (64 * j + lane < kv) ? p[64 * j] : v4i{0, 0, 0, 0};
+    };
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++)
+        if (r0 + d * W < r1)
+            load_row(r0 + d * W, wb[d]);
+
+    v4i xc[MR][KV];
+    if constexpr (DYNQ) {
+        // absmax of a row: non-negative floats order like their bit patterns, so an integer
+        // maximum in LDS collects the waves' shares in any order
+        if (threadIdx.x < MR)
+            s_amax[threadIdx.x] = 0u;
+        lds_barrier();
+#pragma unroll
+        for (int i = 0; i < XV; i++) {
+            const float m = vtlhip::qdev::wave_max(vtlhip::qdev::absmax4(0.0f, xr[i]));
+            if (lane == 0)
+                atomicMax(&s_amax[(i * 512 + (int)threadIdx.x) / PIECES], __float_as_uint(m));
+        }
+        lds_barrier();
+        if (threadIdx.x < MR) {
+            const float sx = __uint_as_float(s_amax[threadIdx.x]) / 127.0f;
+            const vtlhip::qdev::QuantScale qp = vtlhip::qdev::make_quant_scale(sx);
+            s_sa[threadIdx.x] = sx;
+            s_rinv[threadIdx.x] = qp.rinv;
+            s_fast[threadIdx.x] = qp.fast ? 1 : 0;
+        }
+        lds_barrier();
+#pragma unroll
+        for (int i = 0; i < XV; i++) {  // pieces past K and rows past M are written as zeros
+            const int f = i * 512 + (int)threadIdx.x, row = f / PIECES;
+            // one row per wave instruction: scalar values, so the choice of path is a scalar branch
+            vtlhip::qdev::QuantScale qp;
+            qp.scale = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(s_sa[row])));
+            qp.rinv = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(s_rinv[row])));
+            qp.fast = __builtin_amdgcn_readfirstlane(s_fast[row]) != 0;
+            reinterpret_cast<unsigned *>(xq)[f] = vtlhip::qdev::quant4(xr[i], qp);
+        }
+        lds_barrier();
+#pragma unroll
+        for (int m = 0; m < MR; m++)
+#pragma unroll
+            for (int j = 0; j < KV; j++)
+                xc[m][j] = reinterpret_cast<const v4i *>(xq)[m * 64 * KV + 64 * j + lane];
+    } else {
+#pragma unroll
+        for (int m = 0; m < MR; m++) {
+            const v4i *p = reinterpret_cast<const v4i *>(g.A + (int64_t)(m < M ? m : 0) * K) + lane;
+#pragma unroll
+            for (int j = 0; j < KV; j++)
+                xc[m][j] = (m < M && 64 * j + lane < kv) ? p[64 * j] : v4i{0, 0, 0, 0};
+        }
+    }
+
+    const int my_m = lane % MR, my_slot = lane / MR;
+    float sav = 0.0f;
+    if (F32OUT && my_m < M)
+        sav = DYNQ ? s_sa[my_m] : g.sa[my_m * g.sa_stride];
+    int res = 0, it = 0;
+    // scale and bias of the weight row this lane parks next are fetched a batch ahead
+    float swv = 0.0f, bv = 0.0f;
+    auto fetch_scales = [&](int it0) {
+        const int64_t n = r0 + (int64_t)(it0 + my_slot) * W;
+        if (F32OUT && my_m < M && n < r1) {
+            swv = g.sw[n * g.sw_stride];
+            if (g.bias)
+                bv = g.bias[n];
+        }
+    };
+    fetch_scales(0);
+    // weight rows it0 .. it0 + SLOTS - 1 of this wave's sequence are parked: scale and store them
+    auto flush = [&](int it0) {
+        const int64_t n = r0 + (int64_t)(it0 + my_slot) * W;
+        if (my_m < M && n < r1 && it0 + my_slot < it) {
+            const int64_t o = (int64_t)my_m * N + n;
+            if constexpr (F32OUT) {
+                const float sc = sav * swv;
+                float y = (float)res * sc;
+                if (g.bias)
+                    y = y + bv;
+                if (g.relu && y < 0.0f)
+                    y = 0.0f;
+                reinterpret_cast<float *>(g.out)[o] = y;
+            } else {
+                reinterpret_cast<int32_t *>(g.out)[o] = res;
+            }
+        }
+    };
+    for (int64_t rb = r0; rb < r1; rb += RING * W) {
+#pragma unroll
+        for (int u = 0; u < RING; u++) {
+            const int64_t r = rb + u * W;
+            if (r >= r1)
+                break;
+            if (r + DEPTH * W < r1)
+                load_row(r + DEPTH * W, wb[(u + DEPTH) % RING]);
+            int acc[MR];
+#pragma unroll
+            for (int m = 0; m < MR; m++)
+                acc[m] = 0;
+#pragma unroll
+            for (int j = 0; j < KV; j++)
+#pragma unroll
+                for (int c = 0; c < 4; c++)
+#pragma unroll
+                    for (int m = 0; m < MR; m++)
+                        acc[m] = __builtin_amdgcn_sdot4(wb[u][j][c], xc[m][j][c], acc[m], false);
+            const int tot = wave_sum_rows<MR>(acc, lane);
+            res = (my_slot == it % SLOTS) ? tot : res;
+            it++;
+            if (it % SLOTS == 0) {
+                flush(it - SLOTS);
+                fetch_scales(it);
+            }
+        }
+    }
+    if (it % SLOTS != 0)
+        flush(it - it % SLOTS);
+}
 
 
 // Any shape, any alignment: one output per thread.  Only used when K is not a
@@ -1158,6 +1381,85 @@ int launch_gemv(const GemmArgs &g, hipStream_t st)
     return check_launch("linear_gemv_kernel");
 }
 
+// A few tokens (2 <= M <= 8) against a weight matrix of rows up to 1024 * 32 / MR bytes.
+template <int KV, int MR, bool DYNQ, bool F32OUT>
+int launch_gemv_rows_kv(const GemmArgs &g, hipStream_t st)
+{
+    constexpr int NWAVE = 8;
+    // Codes and weight rows live in registers, which limits the waves a SIMD holds; with few
+    // waves a third weight row in flight per wave keeps enough bytes on their way from HBM.
+    constexpr int DEPTH = (MR * KV >= 16 && 4 * KV * (MR + 4) + 40 <= 256) ? 3 : 2;
+    constexpr int REGS = 4 * KV * (MR + DEPTH + 1) + 40;
+    // a workgroup of 8 waves puts two on every SIMD: whole workgroups only
+    constexpr int OCC = 512 / REGS >= 8 ? 8 : (512 / REGS >= 2 ? (512 / REGS) & ~1 : 2);
+    const int rows_per_wave = (g.N + 1024 * OCC - 1) / (1024 * OCC);  // every wave the same number of rows
+    const int64_t waves = (g.N + rows_per_wave - 1) / rows_per_wave;
+    const dim3 grid((unsigned)((waves + NWAVE - 1) / NWAVE)), block(64 * NWAVE);
+    if constexpr (DYNQ && MR * KV > 8) {
+        return VTL_HIP_ERR_UNSUPPORTED;  // not routed here: a quantizer launch of its own is cheaper
+    } else {
+        hipLaunchKernelGGL((linear_gemv_rows_kernel<KV, MR, DEPTH, DYNQ, F32OUT>), grid, block, 0, st, g);
+        return check_launch("linear_gemv_rows_kernel");
+    }
+}
+
+template <int MR, bool DYNQ, bool F32OUT>
+int launch_gemv_rows_mr(const GemmArgs &g, hipStream_t st)
+{
+    const int kv = (g.K + 1023) / 1024;
+    if (kv <= 1)
+        return launch_gemv_rows_kv<1, MR, DYNQ, F32OUT>(g, st);
+    if (kv <= 2)
+        return launch_gemv_rows_kv<2, MR, DYNQ, F32OUT>(g, st);
+    if (kv <= 4)
+        return launch_gemv_rows_kv<4, MR, DYNQ, F32OUT>(g, st);
+    if constexpr (MR <= 4)
+        return launch_gemv_rows_kv<8, MR, DYNQ, F32OUT>(g, st);
+    return VTL_HIP_ERR_UNSUPPORTED;  // not reached: 8 rows are routed here up to K = 4096
+}
+
+template <bool DYNQ, bool F32OUT>
+int launch_gemv_rows(const GemmArgs &g, hipStream_t st)
+{
+    if (g.M <= 2)
+        return launch_gemv_rows_mr<2, DYNQ, F32OUT>(g, st);
+    if (g.M <= 4)
+        return launch_gemv_rows_mr<4, DYNQ, F32OUT>(g, st);
+    return launch_gemv_rows_mr<8, DYNQ, F32OUT>(g, st);
+}
+
+// The codes of the MR rows stay in registers: at most 32 pieces of 16 bytes per lane.
+inline bool gemv_rows_applies(const void *rows, const void *w, int M, int N, int K)
+{
+    return M >= 2 && M <= 8 && K % 16 == 0 && K >= 256 && K <= (M <= 4 ? 8192 : 4096) && aligned16(rows) &&
+           aligned16(w) && !getenv("VTL_HIP_NO_GEMV");
+}
+
+// Where the few-token kernel beats the MFMA weight-streaming kernel (measured, N = 2048 ... 28672,
+// K = 1024 ... 8192): its dot4 work grows with M * N * K while the other's does not, but it has no
+// LDS staging and a lower fixed cost.  Shapes the other kernel cannot take (K % 256 != 0) come here.
+inline bool gemv_rows_faster(int M, int N, int K)
+{
+    if (const char *force = getenv("VTL_HIP_GEMV_ROWS"))   // "1" / "0" force the choice (tests, tuning)
+        return atoi(force) != 0;
+    if (M <= 2 || K % 256 != 0)
+        return true;
+    if (M <= 4)
+        return K >= 2048 || N <= 8192;
+    return (int64_t)N * K <= (K >= 4096 ? (int64_t)24 << 20 : (int64_t)4 << 20);
+}
+
+// Quantizing the rows inside every workgroup of the few-token kernel costs about 15 instructions
+// per element and workgroup; past 8192 elements (rows rounded up to 2, 4 or 8) a quantizer launch
+// of its own is cheaper.
+inline bool gemv_rows_fused_quant_faster(int M, int N, int K)
+{
+    const int mr = M <= 2 ? 2 : (M <= 4 ? 4 : 8);
+    if (const char *force = getenv("VTL_HIP_GEMV_ROWS"))   // only the instantiated sizes can be forced
+        return atoi(force) != 0 && (int64_t)mr * ((K + 1023) / 1024) <= 8;
+    return (int64_t)mr * K <= 8192 && (mr < 8 || (int64_t)N * K <= (int64_t)4 << 20);
+}
+
 // N <= 64 * 4096: a wave parks one sum per lane.
 inline bool gemv_applies(const void *row, const void *w, int N, int K)
 {
@@ -1204,6 +1506,9 @@ int launch_gemm(const GemmArgs &g_in, hipStream_t st)
     if (g.M == 1 && g.K >= 256 && (g.K <= 4096 || g.N < 8192) && gemv_applies(g.A, g.Bt, g.N, g.K) &&
         !getenv("VTL_HIP_GEMM_CONFIG") && !getenv("VTL_HIP_GEMM_SMALL"))
         return launch_gemv<false, F32OUT>(g, st);
+    if (g.N >= 2048 && gemv_rows_applies(g.A, g.Bt, g.M, g.N, g.K) && gemv_rows_faster(g.M, g.N, g.K) &&
+        !getenv("VTL_HIP_GEMM_CONFIG") && !getenv("VTL_HIP_GEMM_SMALL"))
+        return launch_gemv_rows<false, F32OUT>(g, st);
     if (g.K % 256 == 0 && g.M <= 32 && g.N >= 2048 && !getenv("VTL_HIP_GEMM_CONFIG"))
         return launch_skinny<F32OUT>(g, st);  // weight streaming: enough row blocks to fill the chip
     const int64_t t32 = (int64_t)((g.M + 31) / 32) * ((g.N + 31) / 32);
@@ -1298,6 +1603,12 @@ int vtl_hip_linear_f32_dynquant(const float *X, const int8_t *Wq, const float *s
         // VTL_HIP_NO_FUSED_DECODE forces the two-launch path (tests).
         GemmArgs g{nullptr, Wq, Y, nullptr, sw, bias, M, N, K, 1, 1, relu ? 1 : 0, 1, nullptr, X, 0};
         return launch_gemv<true, true>(g, current_stream());
+    }
+    if (N >= 2048 && gemv_rows_applies(X, Wq, M, N, K) && gemv_rows_fused_quant_faster(M, N, K) &&
+        !getenv("VTL_HIP_NO_FUSED_DECODE")) {
+        // a few tokens and short rows: same, each workgroup quantizes the rows itself
+        GemmArgs g{nullptr, Wq, Y, nullptr, sw, bias, M, N, K, 1, 1, relu ? 1 : 0, 1, nullptr, X, 0};
+        return launch_gemv_rows<true, true>(g, current_stream());
     }
     if (!workspace) {   // no caller scratch: stage in the library's own buffer
         workspace = vtlhip::library_workspace(vtl_hip_linear_f32_dynquant_workspace(M, K), 1);
