@@ -261,35 +261,40 @@ def bench_other_configs(timer: Timer, steps: int, warmup: int):
         Ws.append(wq)
         Ss.append(sw)
     X = HipTensor.from_host(rng.standard_normal((m, dims[0]), dtype=np.float32))
-    Ys = [HipTensor.empty([m, dims[i + 1]], np.float32) for i in range(3)]
-    ws = HipStorage.empty(int(capi.lib().vtl_hip_linear_f32_dynquant_workspace(m, max(dims))), np.uint8)
+    # activations travel as per-token int8 codes + row scales: the first layer's input is
+    # quantized, every hidden layer hands codes to the next (epilogue, ReLU and requantization
+    # in one pass over the int32 sums), the last one writes f32
+    Qs = [HipTensor.empty([m, dims[i]], np.int8) for i in range(3)]
+    Sx = [HipTensor.empty([m], np.float32) for i in range(3)]
+    Y = HipTensor.empty([m, dims[3]], np.float32)
+
+    def layer(i):
+        if i == 0:
+            capi.call("vtl_hip_quantize_f32_i8", X.ptr, m, dims[0], 1, Qs[0].ptr, Sx[0].ptr)
+        if i < 2:
+            capi.call("vtl_hip_linear_i8_requant", Qs[i].ptr, Sx[i].ptr, 1, Ws[i].ptr, Ss[i].ptr, 1, None, 1,
+                      Qs[i + 1].ptr, Sx[i + 1].ptr, None, m, dims[i + 1], dims[i])
+        else:
+            capi.call("vtl_hip_linear_i8_f32", Qs[i].ptr, Sx[i].ptr, 1, Ws[i].ptr, Ss[i].ptr, 1, None, Y.ptr,
+                      m, dims[i + 1], dims[i], 0)
 
     def c5():
-        cur = X
         for i in range(3):
-            capi.call("vtl_hip_linear_f32_dynquant", cur.ptr, Ws[i].ptr, Ss[i].ptr, None, Ys[i].ptr, m,
-                      dims[i + 1], dims[i], 1 if i < 2 else 0, ws.ptr, ws.size)
-            cur = Ys[i]
+            layer(i)
     us = timed(c5)
     ops = 2.0 * m * sum(dims[i] * dims[i + 1] for i in range(3))
     wbytes = float(sum(dims[i] * dims[i + 1] for i in range(3)))
     layers = {}
     for i in range(3):
-        src = X if i == 0 else Ys[i - 1]
-
-        def one(i=i, src=src):
-            capi.call("vtl_hip_linear_f32_dynquant", src.ptr, Ws[i].ptr, Ss[i].ptr, None, Ys[i].ptr, m,
-                      dims[i + 1], dims[i], 1 if i < 2 else 0, ws.ptr, ws.size)
-        lus = timed(one)
+        lus = timed(lambda i=i: layer(i))
         layers[f"{dims[i]}->{dims[i + 1]}"] = {"us": lus, "TOPS": 2.0 * m * dims[i] * dims[i + 1] / lus / 1e6,
                                                "weight_GB/s": dims[i] * dims[i + 1] / lus / 1e3}
     out["configs[4] int8 MLP chain 256x4096->11008->4096->1024"] = {
         "us": us, "TOPS": ops / us / 1e6, "weight_GB/s": wbytes / us / 1e3, "ops": ops,
-        "per_layer (row quantize + int8 linear)": layers}
+        "per_layer (input quantize + linear/ReLU/requantize, same, linear to f32)": layers}
     capi.call("vtl_hip_sync")
-    for h in Ws + Ss + Ys + [X]:
+    for h in Ws + Ss + Qs + Sx + [X, Y]:
         h.release()
-    ws.release()
     return out
 
 

@@ -126,6 +126,19 @@ int vtl_hip_linear_i8_f32(const int8_t *A, const float *sa, int sa_per_row,
                           const int8_t *Wq, const float *sw, int sw_per_col,
                           const float *bias, float *Y, int M, int N, int K, int relu);
 
+/* The int8 linear whose output feeds the next quantized layer (Linear -> ReLU
+ * -> Linear with activations requantized per token): y as
+ * vtl_hip_linear_i8_f32 computes it, then every row of y quantized as
+ * vtl_hip_quantize_f32_i8 with per_row = 1 would - codes Yq[M,N], scales
+ * sy[M] - with the bits of those two calls.  Y receives the f32 rows when it
+ * is not NULL.  The activation hand-off between layers of the reference's
+ * device chain (DeviceGpuChain, autograd_cuda/device_session_gpu_d_cuda.v:9-55)
+ * with the requantization that an int8 chain adds. */
+int vtl_hip_linear_i8_requant(const int8_t *A, const float *sa, int sa_per_row,
+                              const int8_t *Wq, const float *sw, int sw_per_col,
+                              const float *bias, int relu, int8_t *Yq, float *sy, float *Y,
+                              int M, int N, int K);
+
 /* Per-token (row) quantization of X[M,K] on the fly, then the int8 linear
  * against per-output-channel quantized weights.  workspace: device scratch
  * of at least vtl_hip_linear_f32_dynquant_workspace(M, K) bytes, 16-byte

@@ -169,6 +169,14 @@ def linear_i8_f32(A, sa, Wq, sw, bias, relu=False, threads: int = 1) -> np.ndarr
     return Y
 
 
+def linear_i8_requant(A, sa, Wq, sw, bias, relu=False, threads: int = 1):
+    """The int8 linear followed by per-row quantization of its f32 output: the
+    hand-off between two int8 layers.  Composition of linear_i8_f32 and quantize."""
+    y = linear_i8_f32(A, sa, Wq, sw, bias, relu=relu, threads=threads)
+    q, s = quantize(y, True, threads=threads)
+    return q, s, y
+
+
 def linear_f32_dynquant(X, Wq, sw, bias, relu=False, threads: int = 1) -> np.ndarray:
     X = _c(X, np.float32)
     Wq = _c(Wq, np.int8)

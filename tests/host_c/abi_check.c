@@ -15,13 +15,15 @@ int main(void)
     int (*gemm)(const int8_t *, const int8_t *, int32_t *, int, int, int) = vtl_hip_gemm_i8_i32;
     int (*linear)(const int8_t *, const float *, int, const int8_t *, const float *, int, const float *, float *,
                   int, int, int, int) = vtl_hip_linear_i8_f32;
+    int (*requant)(const int8_t *, const float *, int, const int8_t *, const float *, int, const float *, int,
+                   int8_t *, float *, float *, int, int, int) = vtl_hip_linear_i8_requant;
     int (*dynquant)(const float *, const int8_t *, const float *, const float *, float *, int, int, int, int,
                     void *, size_t) = vtl_hip_linear_f32_dynquant;
     int (*matmul)(const float *, const float *, float *, int, int, int, int, int) = vtl_hip_matmul_f32;
     int (*backward)(const float *, const float *, const float *, float *, float *, float *, int, int, int) =
         vtl_hip_linear_backward_f32;
     int failures = 0;
-    if (!quantize || !dequantize || !gemm || !linear || !dynquant || !matmul || !backward)
+    if (!quantize || !dequantize || !gemm || !linear || !requant || !dynquant || !matmul || !backward)
         failures++;
     if (strcmp(vtl_hip_strerror(VTL_HIP_OK), "success") != 0)
         failures++;

@@ -67,6 +67,9 @@ def test_bad_arguments_return_status_not_abort():
     assert S("vtl_hip_gemm_i8_i32", one, one, one, -4, 4, 16) == E
     assert S("vtl_hip_gemm_i8_i32", one, one, one, 4, 4, 1 << 20) == capi.ERR_UNSUPPORTED
     assert S("vtl_hip_linear_i8_f32", one, None, 1, one, one, 1, None, one, 4, 4, 16, 0) == E
+    assert S("vtl_hip_linear_i8_requant", one, one, 1, one, one, 1, None, 0, one, None, None, 4, 4, 16) == E   # no scales out
+    assert S("vtl_hip_linear_i8_requant", one, one, 1, one, one, 1, None, 0, None, one, None, 4, 4, 16) == E   # no codes out
+    assert S("vtl_hip_linear_i8_requant", one, one, 1, one, one, 1, None, 0, one, one, None, 0, 4, 16) == capi.OK
     assert S("vtl_hip_linear_f32_dynquant", one, one, one, None, one, 4, 4, 16, 0, C.c_void_p(20), 4096) == E   # misaligned
     assert S("vtl_hip_linear_f32_dynquant", one, one, one, None, one, 4, 4, 16, 0, one, 8) == E
     assert S("vtl_hip_relu_f32", None, 4) == E
@@ -217,6 +220,6 @@ def test_v_binding_declarations_match_the_header():
                 seen.add(name)
     # the binding uses the compute surface of the library
     for must in ("vtl_hip_quantize_f32_i8", "vtl_hip_dequantize_i8_f32", "vtl_hip_gemm_i8_i32", "vtl_hip_linear_i8_f32",
-                 "vtl_hip_linear_f32_dynquant", "vtl_hip_matmul_f32", "vtl_hip_linear_backward_f32",
+                 "vtl_hip_linear_i8_requant", "vtl_hip_linear_f32_dynquant", "vtl_hip_matmul_f32", "vtl_hip_linear_backward_f32",
                  "vtl_hip_malloc", "vtl_hip_free", "vtl_hip_memcpy_h2d", "vtl_hip_memcpy_d2h"):
         assert must in seen, must

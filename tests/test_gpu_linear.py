@@ -5,7 +5,7 @@ import pytest
 
 import oracle
 from helpers import CPU_THREADS, KAT, dev, rel_err
-from vtl_amd import (PER_CHANNEL, PER_TENSOR, HipSession, QuantLinearLayer, Sequential, capi,
+from vtl_amd import (PER_CHANNEL, PER_TENSOR, HipSession, QuantLinearLayer, Sequential, capi, linear_i8_requant_hip,
                      linear_forward_hip_f32, workloads)
 from vtl_amd.tensor import HipTensor, linear_f32_dynquant_hip
 
@@ -62,6 +62,47 @@ def test_decode_linear_config(hip, m):
     assert got.shape == (m, 14336)
     assert rel_err(got, want) <= F32_REL_TOL and np.array_equal(got, want)
     for h in (W, Wq, Sw, X, y):
+        h.release()
+
+
+# the requantizing linear: tile kernel with and without a K split, ragged tiles, every row-kernel
+# size class (N <= 1024 ... 16384), and the shapes that fall back to linear + row quantizer
+# (few rows, N % 4 != 0, N > 16384, K % 16 != 0)
+REQUANT_SHAPES = [(256, 1024, 4096), (256, 4096, 11008), (256, 11008, 4096), (100, 1200, 1360), (64, 2048, 512),
+                  (33, 6000, 256), (40, 16384, 128), (300, 4, 2432), (1000, 512, 64),
+                  (8, 2048, 1024), (32, 300, 512), (64, 1002, 256), (40, 16388, 64), (64, 256, 100)]
+
+
+@pytest.mark.parametrize("mnk", REQUANT_SHAPES)
+def test_requantizing_linear_equals_linear_then_row_quantize(hip, mnk, monkeypatch):
+    """vtl_hip_linear_i8_requant gives the codes, scales and (when asked for) f32 rows of
+    vtl_hip_linear_i8_f32 followed by the per-row quantizer, and of the oracle."""
+    m, n, k = mnk
+    rng = np.random.Generator(np.random.Philox(m * 13 + n * 5 + k))
+    a = rng.integers(-127, 128, (m, k), dtype=np.int8)
+    w = rng.integers(-127, 128, (n, k), dtype=np.int8)
+    sa = (rng.uniform(0.5, 1.5, m) * np.exp(rng.uniform(-10, 10, m)) / 127).astype(np.float32)
+    sw = (rng.uniform(0.5, 1.5, n) / 127).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    A, W, SA, SW, B = dev(a), dev(w), dev(sa), dev(sw), dev(bias)
+    for relu, b_dev, b_host in ((True, B, bias), (False, None, None)):
+        q_ref, s_ref, y_ref = oracle.linear_i8_requant(a, sa, w, sw, b_host, relu=relu, threads=CPU_THREADS)
+        yq, sy, y = linear_i8_requant_hip(A, SA, W, SW, b_dev, relu=relu, keep_f32=True)
+        assert np.array_equal(y.cpu(), y_ref) and np.array_equal(sy.cpu(), s_ref)
+        assert np.array_equal(yq.cpu(), q_ref)
+        yq2, sy2 = linear_i8_requant_hip(A, SA, W, SW, b_dev, relu=relu)       # no f32 rows wanted
+        assert np.array_equal(yq2.cpu(), q_ref) and np.array_equal(sy2.cpu(), s_ref)
+        monkeypatch.setenv("VTL_HIP_NO_FUSED_REQUANT", "1")                    # linear, then row quantizer
+        yq3, sy3 = linear_i8_requant_hip(A, SA, W, SW, b_dev, relu=relu)
+        monkeypatch.delenv("VTL_HIP_NO_FUSED_REQUANT")
+        assert np.array_equal(yq3.cpu(), q_ref) and np.array_equal(sy3.cpu(), s_ref)
+        for h in (yq, sy, y, yq2, sy2, yq3, sy3):
+            h.release()
+    # rows that come out all zero (ReLU of a negative row): scale 0, codes 0
+    neg = dev(np.full(n, -1e30, np.float32))
+    yq, sy = linear_i8_requant_hip(A, SA, W, SW, neg, relu=True)
+    assert not yq.cpu().any() and not sy.cpu().any()
+    for h in (A, W, SA, SW, B, neg, yq, sy):
         h.release()
 
 

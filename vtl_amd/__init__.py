@@ -15,4 +15,5 @@ from .layers import (PER_CHANNEL, PER_TENSOR, HipSession, QuantLinearLayer,  # n
 from .models import Sequential  # noqa: F401
 from .storage import HipParams, HipStorage, hip_available  # noqa: F401
 from .tensor import (HipTensor, colsum_hip, gemm_i8_hip, linear_backward_hip,  # noqa: F401
-                     linear_f32_dynquant_hip, linear_hip, linear_i8_hip, matmul_hip)
+                     linear_f32_dynquant_hip, linear_hip, linear_i8_hip, linear_i8_requant_hip,
+                     matmul_hip)

@@ -46,6 +46,11 @@ struct GemmArgs {
     int32_t *partials;  // [splits][M][N] int32 partial sums when splits > 1
     const float *xf32;  // f32 activations [M,K] for the kernel that quantizes them itself
     int cached_out;     // f32 epilogue of the 256x256 tile: cached instead of non-temporal stores
+    // When set, the launch leaves raw int32 sums in `partials` (also without a K split) and a
+    // row kernel applies the epilogue and quantizes each output row: codes here, row scales in
+    // requant_scales, the f32 rows in `out` unless that is null.
+    int8_t *requant_codes;
+    float *requant_scales;
 };
 
 // LDS tiles are rows of BK bytes (BK/16 chunks of 16 bytes).  The chunk index
@@ -486,7 +491,8 @@ __global__ __launch_bounds__(256) void splitk_finalize_kernel(const GemmArgs g)
 #pragma unroll
     for (int j = 0; j < VEC; j++)
         acc[j] = 0;
-    for (int s = 0; s < g.splits; s++) {
+#pragma unroll 4
+    for (int s = 0; s < g.splits; s++) {   // independent loads: several K ranges in flight per thread
         const int32_t *p = g.partials + (int64_t)s * mn + idx;
         if (VEC == 4) {
             const v4i v = *reinterpret_cast<const v4i *>(p);
@@ -524,6 +530,106 @@ __global__ __launch_bounds__(256) void splitk_finalize_kernel(const GemmArgs g)
             out[0] = acc[0];
         }
     }
+}
+
+// Epilogue and per-row requantization in one pass over the int32 sums: one
+// workgroup per output row adds the K ranges up (exact), applies
+// y = fl(fl(f32(acc) * fl(sa * sw)) + bias) and ReLU as the other epilogues do,
+// keeps the row in registers (4 * NV consecutive-by-four columns per thread,
+// N <= 4 * T * NV, N % 4 == 0), takes its absmax and writes the codes the row
+// quantizer would write for that f32 row (same arithmetic, same bits), its
+// scale, and the f32 row itself when asked for.
+template <int T, int NV>
+__global__ __launch_bounds__(T) void finalize_requant_kernel(const GemmArgs g)
+{
+    constexpr int NW = T / 64;
+    __shared__ float red[NW];
+    const int m = blockIdx.x, N = g.N;
+    const int64_t mn = (int64_t)g.M * N;
+    const float sa = g.sa[(int64_t)m * g.sa_stride];
+    // all loads of a K range are issued before the previous range is added: NV (x2) in flight
+    v4i acc[NV];
+    const int32_t *p0 = g.partials + (int64_t)m * N + 4 * (int)threadIdx.x;
+#pragma unroll
+    for (int v = 0; v < NV; v++)
+        acc[v] = 4 * (v * T + (int)threadIdx.x) < N ? *reinterpret_cast<const v4i *>(p0 + 4 * v * T) : v4i{0, 0, 0, 0};
+#pragma unroll 2
+    for (int s = 1; s < g.splits; s++) {
+        v4i t[NV];
+#pragma unroll
+        for (int v = 0; v < NV; v++)
+            t[v] = 4 * (v * T + (int)threadIdx.x) < N ? *reinterpret_cast<const v4i *>(p0 + (int64_t)s * mn + 4 * v * T)
+                                                      : v4i{0, 0, 0, 0};
+#pragma unroll
+        for (int v = 0; v < NV; v++)
+            acc[v] += t[v];
+    }
+    f4 y[NV];
+    float am = 0.0f;
+#pragma unroll
+    for (int v = 0; v < NV; v++) {
+        const int n = 4 * (v * T + (int)threadIdx.x);
+        y[v] = f4{0.f, 0.f, 0.f, 0.f};
+        if (n < N) {
+            const f4 swv = g.sw_stride ? *reinterpret_cast<const f4 *>(g.sw + n) : f4{g.sw[0], g.sw[0], g.sw[0], g.sw[0]};
+            const f4 bv = g.bias ? *reinterpret_cast<const f4 *>(g.bias + n) : f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float sc = sa * swv[j];
+                float t = (float)acc[v][j] * sc;
+                if (g.bias)
+                    t = t + bv[j];
+                if (g.relu && t < 0.0f)
+                    t = 0.0f;
+                y[v][j] = t;
+            }
+            am = vtlhip::qdev::absmax4(am, y[v]);
+        }
+    }
+    am = vtlhip::qdev::wave_max(am);
+    if ((threadIdx.x & 63) == 0)
+        red[threadIdx.x >> 6] = am;
+    __syncthreads();
+    am = red[0];
+#pragma unroll
+    for (int i = 1; i < NW; i++)
+        am = fmaxf(am, red[i]);
+    const float sy = am / 127.0f;
+    const vtlhip::qdev::QuantScale qp = vtlhip::qdev::make_quant_scale(sy);
+    if (threadIdx.x == 0)
+        g.requant_scales[m] = sy;
+#pragma unroll
+    for (int v = 0; v < NV; v++) {
+        const int n = 4 * (v * T + (int)threadIdx.x);
+        if (n < N) {
+            const int64_t o = (int64_t)m * N + n;
+            *reinterpret_cast<unsigned *>(g.requant_codes + o) = vtlhip::qdev::quant4(y[v], qp);
+            if (g.out)
+                *reinterpret_cast<f4 *>(reinterpret_cast<float *>(g.out) + o) = y[v];
+        }
+    }
+}
+
+inline bool requant_rows_fit(int N)
+{
+    return N % 4 == 0 && N <= 16384;
+}
+
+int launch_finalize_requant(const GemmArgs &g, hipStream_t st)
+{
+    const dim3 grid((unsigned)g.M);
+    // one workgroup per row and often few rows: large workgroups keep more loads in flight
+    if (g.N <= 1024)
+        hipLaunchKernelGGL((finalize_requant_kernel<256, 1>), grid, dim3(256), 0, st, g);
+    else if (g.N <= 2048)
+        hipLaunchKernelGGL((finalize_requant_kernel<512, 1>), grid, dim3(512), 0, st, g);
+    else if (g.N <= 4096)
+        hipLaunchKernelGGL((finalize_requant_kernel<1024, 1>), grid, dim3(1024), 0, st, g);
+    else if (g.N <= 8192)
+        hipLaunchKernelGGL((finalize_requant_kernel<1024, 2>), grid, dim3(1024), 0, st, g);
+    else
+        hipLaunchKernelGGL((finalize_requant_kernel<1024, 4>), grid, dim3(1024), 0, st, g);
+    return check_launch("finalize_requant_kernel");
 }
 
 // Weight-streaming kernel for M <= 32 (decode-shaped linear): bound by reading
@@ -1236,17 +1342,31 @@ int launch_dma(GemmArgs g, int splits, hipStream_t st)
     if (splits < 1)
         splits = 1;
     g.splits = splits;
-    if (splits > 1) {
+    const bool requant = F32OUT && g.requant_codes != nullptr;
+    if (splits > 1 || requant) {
         g.partials = static_cast<int32_t *>(
             vtlhip::library_workspace((size_t)splits * (size_t)g.M * (size_t)g.N * sizeof(int32_t)));
         if (!g.partials)
             return VTL_HIP_ERR_OUT_OF_MEMORY;
     }
-    static PerDevice<bool> done_flags[4];
-    bool *done[4] = {&done_flags[0].get(), &done_flags[1].get(), &done_flags[2].get(), &done_flags[3].get()};
+    static PerDevice<bool> done_flags[6];
+    bool *done[6] = {&done_flags[0].get(), &done_flags[1].get(), &done_flags[2].get(),
+                     &done_flags[3].get(), &done_flags[4].get(), &done_flags[5].get()};
     const bool edge = (g.M % BM) || (g.N % BN) || (g.K % BK);
     g.cached_out = tiles <= 256 ? 1 : 0;  // one round of workgroups
     int rc;
+    if (requant && splits == 1) {
+        // no K split: the int32 sums of the whole K go to the scratch plane the row kernel reads
+        GemmArgs gi = g;
+        gi.out = g.partials;
+        if (edge)
+            rc = launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, false, true, false>, *done[4], lds,
+                                 tiles, 64 * WR * WC, gi, st, "gemm_i8_dma_kernel");
+        else
+            rc = launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, false, false, false>, *done[5], lds,
+                                 tiles, 64 * WR * WC, gi, st, "gemm_i8_dma_kernel");
+        return rc != VTL_HIP_OK ? rc : launch_finalize_requant(g, st);
+    }
     // the partial sums of a split launch are int32 whatever the final type is
     if (splits > 1 && edge)
         rc = launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, false, true, true>, *done[0], lds,
@@ -1262,6 +1382,8 @@ int launch_dma(GemmArgs g, int splits, hipStream_t st)
                              tiles, 64 * WR * WC, g, st, "gemm_i8_dma_kernel");
     if (rc != VTL_HIP_OK || splits == 1)
         return rc;
+    if (requant)
+        return launch_finalize_requant(g, st);
     const int64_t mn = (int64_t)g.M * g.N;
     if (g.N % 4 == 0 && aligned16(g.out) && aligned16(g.partials)) {
         hipLaunchKernelGGL((splitk_finalize_kernel<F32OUT, 4>), dim3((unsigned)((mn / 4 + 255) / 256)), dim3(256), 0,
@@ -1570,6 +1692,44 @@ int vtl_hip_linear_i8_f32(const int8_t *A, const float *sa, int sa_per_row, cons
         return VTL_HIP_ERR_UNSUPPORTED;  // la.matmul rejects empty inner dimensions as well
     GemmArgs g{A, Wq, Y, sa, sw, bias, M, N, K, sa_per_row ? 1 : 0, sw_per_col ? 1 : 0, relu ? 1 : 0, 1, nullptr, nullptr, 0};
     return launch_gemm<true>(g, current_stream());
+}
+
+int vtl_hip_linear_i8_requant(const int8_t *A, const float *sa, int sa_per_row, const int8_t *Wq,
+                              const float *sw, int sw_per_col, const float *bias, int relu, int8_t *Yq,
+                              float *sy, float *Y, int M, int N, int K)
+{
+    int st = check_gemm_args(A, Wq, Yq, M, N, K);
+    if (st != VTL_HIP_OK)
+        return st;
+    if (!sa || !sw || !sy)
+        return VTL_HIP_ERR_INVALID_ARG;
+    if (M == 0 || N == 0)
+        return VTL_HIP_OK;
+    if (K == 0)
+        return VTL_HIP_ERR_UNSUPPORTED;
+    GemmArgs g{A, Wq, Y, sa, sw, bias, M, N, K, sa_per_row ? 1 : 0, sw_per_col ? 1 : 0, relu ? 1 : 0, 1, nullptr, nullptr, 0};
+    if (M > 32 && K % 16 == 0 && aligned16(A) && aligned16(Wq) && requant_rows_fit(N) && aligned16(Yq) &&
+        (!Y || aligned16(Y)) && (!sw_per_col || aligned16(sw)) && (!bias || aligned16(bias)) &&
+        !getenv("VTL_HIP_NO_FUSED_REQUANT")) {
+        // tile kernel leaves int32 sums, one row kernel does epilogue + quantization
+        g.requant_codes = Yq;
+        g.requant_scales = sy;
+        int idx, splits;
+        choose_config(M, N, K, idx, splits);
+        return launch_config<true>(idx, g, splits, current_stream());
+    }
+    // any other shape: the f32 rows (in the library's staging buffer when the caller wants none),
+    // then the row quantizer
+    if (!Y) {
+        Y = static_cast<float *>(vtlhip::library_workspace((size_t)M * (size_t)N * sizeof(float), 1));
+        if (!Y)
+            return VTL_HIP_ERR_OUT_OF_MEMORY;
+        g.out = Y;
+    }
+    st = launch_gemm<true>(g, current_stream());
+    if (st != VTL_HIP_OK)
+        return st;
+    return launch_quantize_rows(Y, M, N, Yq, sy, current_stream());
 }
 
 size_t vtl_hip_linear_f32_dynquant_workspace(int M, int K)

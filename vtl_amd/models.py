@@ -4,7 +4,8 @@ mirror of nn/models/sequential.v:52-220 for input / linear / relu / forward.
 `linear(n)` takes its input width from the previous layer
 (nn/models/sequential_info.v:53-60); `forward` loops over the layers
 (sequential.v:204-215).  Between Linear layers the activations stay on the
-device and ReLU is folded into the producing Linear's epilogue, in the spirit
+device, as per-token int8 codes when the next layer is a Linear again, and ReLU
+is folded into the producing Linear's epilogue, in the spirit
 of the reference's GPU activation chain
 (autograd_cuda/device_session_gpu_d_cuda.v:88-181).
 """
@@ -14,7 +15,7 @@ import numpy as np
 
 from .layers import PER_CHANNEL, HipSession, QuantLinearLayer, kaiming_normal
 from .storage import HipParams
-from .tensor import HipTensor
+from .tensor import HipTensor, linear_i8_hip, linear_i8_requant_hip
 
 
 class Sequential:
@@ -54,17 +55,38 @@ class Sequential:
         x = np.asarray(x, np.float32)
         if x.ndim != 2:
             raise ValueError("Matrix expected")
-        cur = HipTensor.from_host(x, self.params)
+        cur = HipTensor.from_host(x, self.params)   # f32 activations, or None while they exist as codes
+        cur_q = None                                # (codes, row scales) between two int8 layers
         try:
             i, n = 0, len(self.layers)
             while i < n:
                 kind = self.layers[i][0]
                 if kind == "linear":
+                    layer = self.layers[i][1]
                     fuse = i + 1 < n and self.layers[i + 1][0] == "relu"
-                    nxt = self.layers[i][1].forward_device(cur, relu=fuse, session=self.session)
-                    cur.release()
-                    cur = nxt
-                    i += 2 if fuse else 1
+                    j = i + (2 if fuse else 1)
+                    feeds_linear = self.mode == PER_CHANNEL and j < n and self.layers[j][0] == "linear"
+                    if cur_q is None and not feeds_linear:
+                        nxt = layer.forward_device(cur, relu=fuse, session=self.session)
+                        cur.release()
+                        cur = nxt
+                    else:
+                        # per-token codes go from layer to layer; the f32 rows in between are
+                        # never written (same bits as quantizing them in a pass of its own)
+                        if cur_q is None:
+                            cur_q = cur.quantize_i8(0)
+                            cur.release()
+                            cur = None
+                        qw = layer.quantized()
+                        if feeds_linear:
+                            nxt_q = linear_i8_requant_hip(cur_q[0], cur_q[1], qw.w_q, qw.sw, qw.bias, relu=fuse)
+                        else:
+                            cur = linear_i8_hip(cur_q[0], cur_q[1], qw.w_q, qw.sw, qw.bias, relu=fuse)
+                            nxt_q = None
+                        for t in cur_q:
+                            t.release()
+                        cur_q = nxt_q
+                    i = j
                 elif kind == "relu":
                     cur.relu_()
                     i += 1
@@ -72,7 +94,11 @@ class Sequential:
                     i += 1
             return cur.cpu()
         finally:
-            cur.release()
+            if cur is not None:
+                cur.release()
+            if cur_q is not None:
+                for t in cur_q:
+                    t.release()
 
     def release(self) -> None:
         for l in self.layers:

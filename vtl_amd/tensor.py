@@ -221,6 +221,29 @@ def linear_i8_hip(x_q: HipTensor, sx: HipTensor, w_q: HipTensor, sw: HipTensor,
     return y
 
 
+def linear_i8_requant_hip(x_q: HipTensor, sx: HipTensor, w_q: HipTensor, sw: HipTensor,
+                          bias: HipTensor | None, relu: bool = False, keep_f32: bool = False):
+    """`linear_i8_requant_hip(x_q, sx, w_q, sw, bias, relu) !(&HipTensor[i8], &HipTensor[f32])`:
+    the int8 linear whose f32 rows are quantized per row for the next int8 layer in the
+    same pass (the bits of linear_i8_hip followed by quantize_i8(0)).  With keep_f32 the
+    f32 output is returned as a third tensor."""
+    x_q._assert(np.int8, what="linear_i8_requant_hip x_q")
+    w_q._assert(np.int8, what="linear_i8_requant_hip w_q")
+    M, N, K = _matmul_shapes(x_q, w_q)
+    if sx.size not in (1, M) or sw.size not in (1, N):
+        raise ValueError("linear_i8_requant_hip: scale sizes do not match the operands")
+    if bias is not None and bias.size != N:
+        raise ValueError(f"linear_i8_requant_hip: bias has {bias.size} entries, expected {N}")
+    params = HipParams(x_q.data.device_id)
+    y_q = HipTensor.empty([M, N], np.int8, params)
+    sy = HipTensor.empty([M], np.float32, params)
+    y = HipTensor.empty([M, N], np.float32, params) if keep_f32 else None
+    capi.call("vtl_hip_linear_i8_requant", x_q.ptr, sx.ptr, int(sx.size == M), w_q.ptr, sw.ptr,
+              int(sw.size == N), bias.ptr if bias is not None else None, int(relu), y_q.ptr, sy.ptr,
+              y.ptr if y is not None else None, M, N, K)
+    return (y_q, sy, y) if keep_f32 else (y_q, sy)
+
+
 def linear_f32_dynquant_hip(x: HipTensor, w_q: HipTensor, sw: HipTensor, bias: HipTensor | None,
                             relu: bool = False, workspace: HipStorage | None = None) -> HipTensor:
     """Per-token quantization of x on the fly, then the int8 linear."""
