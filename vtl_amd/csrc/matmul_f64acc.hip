@@ -482,15 +482,17 @@ int matmul_impl(const T *a, const T *b, T *c, const T *bias, int m, int n, int k
     // Tile choice by a per-compute-unit estimate, in units of one 128x128 tile at
     // peak: a compute unit runs two big workgroups together at ~0.84 of peak and
     // a single one at ~0.75; the 64x64 tile kernel reaches 0.72 (four workgroups
-    // per compute unit) to 0.80 (nine and more) and quantizes four times finer
-    // over the 256 compute units.  Constants fitted to measured times.
+    // per compute unit) to 0.78 (many) and quantizes four times finer over the
+    // 256 compute units.  Constants fitted to measured times (with many tiles
+    // the big one is 7-12 % faster, e.g. 11008x4096x256: 350 against 377 us).
     const int64_t big = (int64_t)((m + 127) / 128) * ((n + 127) / 128);
     const int64_t small = (int64_t)((m + 63) / 64) * ((n + 63) / 64);
     const int64_t c128 = (big + 255) / 256, c64 = (small + 255) / 256;
     const double t128 = (double)(c128 / 2) * (2.0 / 0.84) + (double)(c128 % 2) * (1.0 / 0.75);
-    const double t64 = (double)c64 * 0.25 / (0.84 - 0.48 / (double)c64);
+    const double t64 = (double)c64 * 0.25 / (0.78 - 0.24 / (double)c64);
     // eight waves of 32x64 per 128x128 tile measured a few percent above four waves of 64x64
-    if (t128 <= t64)
+    const char *tile_env = getenv("VTL_HIP_MATMUL_TILE");   // "128" / "64" force the tile (tuning, tests)
+    if (tile_env ? atoi(tile_env) == 128 : t128 <= t64)
         return launch_tile<T, 2, 4, 4, 2>(g, trans_a != 0, trans_b != 0, st);
     const char *force = getenv("VTL_HIP_MATMUL_SPLITS");   // tuning and tests
     // Too few big tiles for the chip but a long K: cut K until about 512 big
