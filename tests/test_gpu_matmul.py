@@ -104,6 +104,25 @@ def test_split_k_paths(hip, dt, monkeypatch):
         t.release()
 
 
+@pytest.mark.parametrize("tile", ["64", "128"])
+def test_forced_tile_sizes(hip, tile, monkeypatch):
+    """VTL_HIP_MATMUL_TILE forces the 64x64 or the 128x128 tile kernel: whole and ragged
+    tiles, all four layouts, both give the oracle's result (integers bit for bit)."""
+    monkeypatch.setenv("VTL_HIP_MATMUL_TILE", tile)
+    rng = np.random.default_rng(int(tile))
+    for (M, N, K, ta, tb) in [(256, 384, 128, False, True), (300, 200, 96, True, False), (129, 65, 260, True, True),
+                              (1, 1, 1, False, False), (640, 512, 64, False, False)]:
+        A = rng.standard_normal((K, M) if ta else (M, K)).astype(np.float32)
+        B = rng.standard_normal((N, K) if tb else (K, N)).astype(np.float32)
+        got = run_matmul(A, B, ta, tb)
+        want = oracle.matmul(A, B, ta, tb, threads=CPU_THREADS)
+        absprod = np.abs(A.T if ta else A).astype(np.float64) @ np.abs(B.T if tb else B).astype(np.float64)
+        assert_close_to_oracle(got, want, absprod)
+        Ai, Bi = np.rint(A * 4).astype(np.float32), np.rint(B * 4).astype(np.float32)
+        exact = (Ai.T if ta else Ai).astype(np.float64) @ (Bi.T if tb else Bi).astype(np.float64)
+        assert np.array_equal(run_matmul(Ai, Bi, ta, tb), exact.astype(np.float32))
+
+
 def test_reference_literals(hip):
     # la/la_test.v:30-37
     a = np.array([[1.0, 0], [0.0, 1]])
