@@ -104,3 +104,37 @@ def test_linear_output_beyond_2_31_elements(hip):
     del rows
     for h in (A, W, SA, SW, B, Y, C):
         h.release()
+
+
+@pytest.mark.parametrize("keep_f32", [False, True])
+def test_requantizing_linear_beyond_2_31_elements(hip, keep_f32):
+    """[140000, 64] x [16384, 64]^T handed on as codes: 2.29e9 outputs.  Without the f32 rows
+    the int32 sums go through 9 GB of library scratch and the row kernel; with them the
+    library takes the two-pass route through the caller's Y.  Sampled row bands against
+    the oracle."""
+    from vtl_amd.tensor import linear_i8_requant_hip
+    m, n, k = 140000, 16384, 64
+    rng = np.random.default_rng(33)
+    a = rng.integers(-127, 128, (m, k), dtype=np.int8)
+    w = rng.integers(-127, 128, (n, k), dtype=np.int8)
+    sa = rng.uniform(0.5, 1.5, m).astype(np.float32)
+    sw = rng.uniform(0.5, 1.5, n).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    assert m * n > 2 ** 31
+    A, W, SA, SW, B = dev(a), dev(w), dev(sa), dev(sw), dev(bias)
+    print("requant", m, n, k, keep_f32, flush=True)
+    out = linear_i8_requant_hip(A, SA, W, SW, B, relu=True, keep_f32=keep_f32)
+    yq, sy = out[0], out[1]
+    scales = sy.cpu()
+    for r0 in (0, 70001, m - 8):
+        band = slice(r0, r0 + 8)
+        got = np.empty((8, n), np.int8)
+        capi.call("vtl_hip_memcpy_d2h", got.ctypes.data, yq.ptr + r0 * n, got.nbytes)
+        q_ref, s_ref, y_ref = oracle.linear_i8_requant(a[band], sa[band], w, sw, bias, relu=True, threads=CPU_THREADS)
+        assert np.array_equal(got, q_ref) and np.array_equal(scales[band], s_ref), f"rows {r0}..{r0 + 8}"
+        if keep_f32:
+            gy = np.empty((8, n), np.float32)
+            capi.call("vtl_hip_memcpy_d2h", gy.ctypes.data, out[2].ptr + r0 * n * 4, gy.nbytes)
+            assert np.array_equal(gy, y_ref)
+    for h in (A, W, SA, SW, B) + tuple(out):
+        h.release()

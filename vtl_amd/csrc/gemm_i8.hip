@@ -1710,6 +1710,9 @@ int vtl_hip_linear_i8_requant(const int8_t *A, const float *sa, int sa_per_row, 
     GemmArgs g{A, Wq, Y, sa, sw, bias, M, N, K, sa_per_row ? 1 : 0, sw_per_col ? 1 : 0, relu ? 1 : 0, 1, nullptr, nullptr, 0};
     if (M > 32 && K % 16 == 0 && aligned16(A) && aligned16(Wq) && requant_rows_fit(N) && aligned16(Yq) &&
         (!Y || aligned16(Y)) && (!sw_per_col || aligned16(sw)) && (!bias || aligned16(bias)) &&
+        // a caller who wants the f32 rows anyway provides the staging: past 256 MiB of int32 sums
+        // the two-pass route through Y needs no scratch of the library's
+        !(Y && (size_t)M * (size_t)N * sizeof(int32_t) > ((size_t)256 << 20)) &&
         !getenv("VTL_HIP_NO_FUSED_REQUANT")) {
         // tile kernel leaves int32 sums, one row kernel does epilogue + quantization
         g.requant_codes = Yq;
