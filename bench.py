@@ -229,6 +229,12 @@ def bench_other_configs(timer: Timer, steps: int, warmup: int):
     W = HipTensor.from_host(rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02))
     Wq, Sw = W.quantize_i8(0)                      # one scale per output channel
     W.release()
+    # The 58.7 MB of codes stay in the 256 MB last-level cache from one launch to the next.
+    # A model's decode step walks through many such matrices, so the same call is also timed
+    # over 12 copies taken in turn (705 MB): every launch then streams its weights from HBM.
+    copies = [Wq] + [HipTensor.empty([n, k], np.int8) for _ in range(11)]
+    for c in copies[1:]:
+        capi.call("vtl_hip_memcpy_d2d", c.ptr, Wq.ptr, n * k)
     dec = {}
     for m in (1, 8, 32, 128):
         X = HipTensor.from_host(rng.standard_normal((m, k), dtype=np.float32))
@@ -239,15 +245,25 @@ def bench_other_configs(timer: Timer, steps: int, warmup: int):
         def c4():
             capi.call("vtl_hip_linear_f32_dynquant", X.ptr, Wq.ptr, Sw.ptr, None, Y.ptr, m, n, k, 0, ws.ptr, ws.size)
         us = timed(c4)
+        turn = [0]
+
+        def c4_streaming():
+            w = copies[turn[0] % len(copies)]
+            turn[0] += 1
+            capi.call("vtl_hip_linear_f32_dynquant", X.ptr, w.ptr, Sw.ptr, None, Y.ptr, m, n, k, 0, ws.ptr, ws.size)
+        us_hbm = timed(c4_streaming)
         algo = n * k + 16384.0 * m + 57344.0 * m + 57344.0     # Wq + X f32 + Y f32 + sw
         dec[f"M={m}"] = {"us": us, "GB/s": algo / us / 1e3, "frac_of_hbm_peak": algo / us / 1e3 / PEAK_HBM_GBPS,
-                         "TOPS": 2.0 * m * n * k / us / 1e6, "algorithmic_bytes": algo}
+                         "TOPS": 2.0 * m * n * k / us / 1e6, "algorithmic_bytes": algo,
+                         "weights_from_hbm": {"us": us_hbm, "GB/s": algo / us_hbm / 1e3,
+                                              "frac_of_hbm_peak": algo / us_hbm / 1e3 / PEAK_HBM_GBPS}}
         capi.call("vtl_hip_sync")
         for h in (X, Y):
             h.release()
         ws.release()
     out["configs[3] decode linear K=4096 N=14336 (quantize on the fly + int8 linear)"] = dec
-    Wq.release()
+    for c in copies:
+        c.release()
     Sw.release()
 
     # configs[4]: 256x4096 -> 11008 -> ReLU -> 4096 -> ReLU -> 1024, device-resident chain
