@@ -1402,9 +1402,9 @@ struct TileConfig {
     int wgs_per_cu;     // workgroups that fit a compute unit's LDS together
 };
 constexpr TileConfig kTileConfigs[] = {
-    {32, 64, 380.f, 1}, {32, 128, 520.f, 2}, {64, 128, 600.f, 2}, {128, 128, 1000.f, 2},
-    {128, 128, 800.f, 1},  // four stages: alone on its compute unit, for launches of one round
-    {256, 256, 2200.f, 1}};
+    {32, 64, 420.f, 1}, {32, 128, 520.f, 2}, {64, 128, 640.f, 2}, {128, 128, 850.f, 2},
+    {128, 128, 750.f, 1},  // four stages: alone on its compute unit, for launches of one round
+    {256, 256, 1800.f, 1}};
 constexpr int kNumTileConfigs = 6;
 
 template <bool F32OUT>
@@ -1426,7 +1426,8 @@ int launch_config(int idx, const GemmArgs &g, int splits, hipStream_t st)
 //   throughput: all K steps of all workgroups x step cost / 256 compute units
 // plus, for split K, the extra launch and the pass over the partial sums.
 // The constants were fitted (random search, least mean log regret) to an
-// exhaustive timing sweep of every tile and split count over 39 shapes.
+// exhaustive timing sweep of every tile and split count over 55 shapes (mean
+// regret 1 %, worst 10 %).
 void choose_config(int M, int N, int K, int &best_idx, int &best_splits)
 {
     const int kt_all = (K + 127) / 128;
@@ -1443,11 +1444,11 @@ void choose_config(int M, int N, int K, int &best_idx, int &best_splits)
                 break;
             const int64_t rounds = (tiles * s + 256 * c.wgs_per_cu - 1) / (256 * c.wgs_per_cu);
             const int steps = (kt_all + s - 1) / s;
-            const float latency = (float)rounds * ((float)steps * c.step_cycles + 4000.f);
-            const float throughput = (float)tiles * (float)s * (float)steps * c.step_cycles / 256.f + 4000.f;
+            const float latency = (float)rounds * ((float)steps * c.step_cycles + 6000.f);
+            const float throughput = (float)tiles * (float)s * (float)steps * c.step_cycles / 256.f + 6000.f;
             float cost = latency > throughput ? latency : throughput;
             if (s > 1)
-                cost += 4500.f + (float)s * (float)M * (float)N * 4.0f / 1500.f;
+                cost += 4500.f + (float)s * (float)M * (float)N * 4.0f / 1000.f;
             if (cost < best) {
                 best = cost;
                 best_idx = i;
