@@ -227,7 +227,9 @@ def test_every_kernel_family_matches_oracle(hip, mnk):
 FEW_TOKEN_SHAPES = [(2, 2048, 256), (2, 3001, 1008), (2, 2050, 2048), (2, 2048, 4096), (2, 2049, 8192),
                     (3, 2048, 1024), (4, 4099, 1040), (4, 2048, 4096), (3, 2051, 8192), (4, 2048, 5120),
                     (5, 2048, 512), (8, 2050, 2032), (7, 2048, 4096), (6, 5000, 3088), (8, 40000, 256),
-                    (2, 140000, 272), (4, 70001, 256), (8, 70001, 256), (5, 140000, 256)]
+                    (2, 140000, 272), (4, 70001, 256), (8, 70001, 256), (5, 140000, 256),
+                    # few weight rows: fewer rows than waves, a single row, ragged everything
+                    (2, 1, 256), (3, 7, 4096), (8, 64, 1024), (4, 100, 8192), (7, 1000, 272), (2, 1536, 4096)]
 
 
 @pytest.mark.parametrize("rows_kernel", ["1", "0", None])

@@ -179,7 +179,8 @@ def test_session_reuses_buffers_on_second_forward(hip):
 @pytest.mark.parametrize("mnk", [(2, 2048, 256), (2, 3001, 1008), (2, 2050, 2048), (2, 2048, 4096), (2, 2064, 3088),
                                  (3, 2048, 1024), (4, 4099, 1040), (4, 2048, 2048), (3, 2051, 272),
                                  (5, 2048, 512), (8, 2050, 1024), (7, 9000, 1008), (6, 2048, 16 * 17),
-                                 (8, 70001, 256)])
+                                 (8, 70001, 256), (2, 1, 256), (3, 7, 2048), (8, 64, 1024), (4, 100, 272),
+                                 (2, 1536, 4096)])
 def test_few_token_fused_decode_equals_two_launch_path(hip, mnk, monkeypatch):
     """2 to 8 tokens with short rows take the few-token kernel whose workgroups quantize the
     rows themselves (forced here for every size it is built for); it must give the bits of

@@ -1558,14 +1558,14 @@ inline bool gemv_rows_applies(const void *rows, const void *w, int M, int N, int
            aligned16(w) && !getenv("VTL_HIP_NO_GEMV");
 }
 
-// Where the few-token kernel beats the MFMA weight-streaming kernel (measured, N = 2048 ... 28672,
-// K = 1024 ... 8192): its dot4 work grows with M * N * K while the other's does not, but it has no
+// Where the few-token kernel beats the MFMA weight-streaming kernel (measured, N = 64 ... 28672,
+// K = 256 ... 8192): its dot4 work grows with M * N * K while the other's does not, but it has no
 // LDS staging and a lower fixed cost.  Shapes the other kernel cannot take (K % 256 != 0) come here.
 inline bool gemv_rows_faster(int M, int N, int K)
 {
     if (const char *force = getenv("VTL_HIP_GEMV_ROWS"))   // "1" / "0" force the choice (tests, tuning)
         return atoi(force) != 0;
-    if (M <= 2 || K % 256 != 0)
+    if (M <= 2 || K % 256 != 0 || N < 2048)   // few weight rows: never slower, 1.8x faster from K = 4096 on
         return true;
     if (M <= 4)
         return K >= 2048 || N <= 8192;
@@ -1629,7 +1629,7 @@ int launch_gemm(const GemmArgs &g_in, hipStream_t st)
     if (g.M == 1 && g.K >= 256 && (g.K <= 4096 || g.N < 8192) && gemv_applies(g.A, g.Bt, g.N, g.K) &&
         !getenv("VTL_HIP_GEMM_CONFIG") && !getenv("VTL_HIP_GEMM_SMALL"))
         return launch_gemv<false, F32OUT>(g, st);
-    if (g.N >= 2048 && gemv_rows_applies(g.A, g.Bt, g.M, g.N, g.K) && gemv_rows_faster(g.M, g.N, g.K) &&
+    if (gemv_rows_applies(g.A, g.Bt, g.M, g.N, g.K) && gemv_rows_faster(g.M, g.N, g.K) &&
         !getenv("VTL_HIP_GEMM_CONFIG") && !getenv("VTL_HIP_GEMM_SMALL"))
         return launch_gemv_rows<false, F32OUT>(g, st);
     if (g.K % 256 == 0 && g.M <= 32 && g.N >= 2048 && !getenv("VTL_HIP_GEMM_CONFIG"))
@@ -1768,7 +1768,7 @@ int vtl_hip_linear_f32_dynquant(const float *X, const int8_t *Wq, const float *s
         GemmArgs g{nullptr, Wq, Y, nullptr, sw, bias, M, N, K, 1, 1, relu ? 1 : 0, 1, nullptr, X, 0};
         return launch_gemv<true, true>(g, current_stream());
     }
-    if (N >= 2048 && gemv_rows_applies(X, Wq, M, N, K) && gemv_rows_fused_quant_faster(M, N, K) &&
+    if (gemv_rows_applies(X, Wq, M, N, K) && gemv_rows_fused_quant_faster(M, N, K) &&
         !getenv("VTL_HIP_NO_FUSED_DECODE")) {
         // a few tokens and short rows: same, each workgroup quantizes the rows itself
         GemmArgs g{nullptr, Wq, Y, nullptr, sw, bias, M, N, K, 1, 1, relu ? 1 : 0, 1, nullptr, X, 0};
