@@ -169,6 +169,7 @@ def test_square_gemm_config_full_size(hip):
 # (few output tiles, long K) with uneven K ranges, and the register-staged
 # tile kernel (K % 128 != 0).
 ROUTED_SHAPES = [(1, 2048, 256), (1, 5, 256), (1, 4099, 4080), (1, 9000, 5120), (1, 300, 8192), (1, 2048, 8448),
+                 (1, 9000, 9232), (1, 4097, 11264), (1, 8192, 14336), (1, 100, 14352), (1, 3000, 16384),
                  (1, 262200, 256),      # more rows than the matrix-vector kernel deals out
 
                  (3, 2050, 256), (8, 2048, 4096), (9, 2048, 768), (16, 2047, 1280),

@@ -221,10 +221,10 @@ def test_few_token_fused_decode_equals_two_launch_path(hip, mnk, monkeypatch):
 
 @pytest.mark.parametrize("nk", [(2048, 256), (2050, 512), (3001, 4096), (2077, 1280), (1, 16), (7, 48), (300, 784),
                                 (14336, 4080), (4097, 5120), (2048, 8192), (1000, 7168), (2050, 8208),
-                                (64, 11008)])
+                                (64, 11008), (2050, 9232), (4096, 11008), (300, 11280), (1000, 14336), (70, 14352)])
 def test_single_token_fused_decode_equals_two_launch_path(hip, nk, monkeypatch):
     """M = 1 takes the matrix-vector kernel that quantizes the token itself (rows of
-    up to 8192 codes, any multiple of 16; longer rows take two launches); it must
+    up to 14336 codes, any multiple of 16; longer rows take two launches); it must
     give the bits of the quantize-then-linear path and of the oracle."""
     n, k = nk
     rng = np.random.Generator(np.random.Philox(n + k))

@@ -1483,13 +1483,16 @@ int launch_skinny(const GemmArgs &g, hipStream_t st)
     return launch_skinny_cfg<2, 2, 4, F32OUT>(g, st);
 }
 
-// Single-token linear (M = 1, K % 16 == 0, K <= 8192, operands 16-byte aligned).
+// Single-token linear (M = 1, K % 16 == 0, K <= 14336, operands 16-byte aligned).
 template <bool DYNQ, bool F32OUT>
 int launch_gemv(const GemmArgs &g, hipStream_t st)
 {
     constexpr int NWAVE = 8;
-    // about sixteen waves per compute unit, and every wave the same number of rows
-    const int rows_per_wave = (g.N + 4095) / 4096;
+    // every wave the same number of rows, and no more waves than the chip holds at once: sixteen
+    // per compute unit up to 6144 codes a row, eight beyond (the codes and three weight rows of a
+    // wave take 150 to 250 registers then)
+    const int max_waves = g.K <= 6144 ? 4096 : 2048;
+    const int rows_per_wave = (g.N + max_waves - 1) / max_waves;
     const int64_t waves = (g.N + rows_per_wave - 1) / rows_per_wave;
     const dim3 grid((unsigned)((waves + NWAVE - 1) / NWAVE)), block(64 * NWAVE);
     switch ((g.K + 1023) / 1024) {
@@ -1499,7 +1502,12 @@ int launch_gemv(const GemmArgs &g, hipStream_t st)
     case 4: hipLaunchKernelGGL((linear_gemv_kernel<4, NWAVE, DYNQ, F32OUT>), grid, block, 0, st, g); break;
     case 5:
     case 6: hipLaunchKernelGGL((linear_gemv_kernel<6, NWAVE, DYNQ, F32OUT>), grid, block, 0, st, g); break;
-    default: hipLaunchKernelGGL((linear_gemv_kernel<8, NWAVE, DYNQ, F32OUT>), grid, block, 0, st, g); break;
+    case 7:
+    case 8: hipLaunchKernelGGL((linear_gemv_kernel<8, NWAVE, DYNQ, F32OUT>), grid, block, 0, st, g); break;
+    case 9:
+    case 10:
+    case 11: hipLaunchKernelGGL((linear_gemv_kernel<11, NWAVE, DYNQ, F32OUT>), grid, block, 0, st, g); break;
+    default: hipLaunchKernelGGL((linear_gemv_kernel<14, NWAVE, DYNQ, F32OUT>), grid, block, 0, st, g); break;
     }
     return check_launch("linear_gemv_kernel");
 }
@@ -1586,7 +1594,7 @@ inline bool gemv_rows_fused_quant_faster(int M, int N, int K)
 // N <= 64 * 4096: a wave parks one sum per lane.
 inline bool gemv_applies(const void *row, const void *w, int N, int K)
 {
-    return K % 16 == 0 && K <= 8192 && N <= 64 * 4096 && aligned16(row) && aligned16(w) && !getenv("VTL_HIP_NO_GEMV");
+    return K % 16 == 0 && K <= 14336 && N <= 64 * 4096 && aligned16(row) && aligned16(w) && !getenv("VTL_HIP_NO_GEMV");
 }
 
 template <bool F32OUT>
@@ -1624,9 +1632,8 @@ int launch_gemm(const GemmArgs &g_in, hipStream_t st)
         g.Bt = ws + a_bytes;
         g.K = Kp;
     }
-    // one row: matrix-vector product (very short rows go to the small-product kernel; long rows
-    // of a tall matrix measured a few percent better in the MFMA weight-streaming kernel)
-    if (g.M == 1 && g.K >= 256 && (g.K <= 4096 || g.N < 8192) && gemv_applies(g.A, g.Bt, g.N, g.K) &&
+    // one row: matrix-vector product (very short rows go to the small-product kernel)
+    if (g.M == 1 && g.K >= 256 && gemv_applies(g.A, g.Bt, g.N, g.K) &&
         !getenv("VTL_HIP_GEMM_CONFIG") && !getenv("VTL_HIP_GEMM_SMALL"))
         return launch_gemv<false, F32OUT>(g, st);
     if (gemv_rows_applies(g.A, g.Bt, g.M, g.N, g.K) && gemv_rows_faster(g.M, g.N, g.K) &&
