@@ -230,7 +230,9 @@ FEW_TOKEN_SHAPES = [(2, 2048, 256), (2, 3001, 1008), (2, 2050, 2048), (2, 2048, 
                     (5, 2048, 512), (8, 2050, 2032), (7, 2048, 4096), (6, 5000, 3088), (8, 40000, 256),
                     (2, 140000, 272), (4, 70001, 256), (8, 70001, 256), (5, 140000, 256),
                     # few weight rows: fewer rows than waves, a single row, ragged everything
-                    (2, 1, 256), (3, 7, 4096), (8, 64, 1024), (4, 100, 8192), (7, 1000, 272), (2, 1536, 4096)]
+                    (2, 1, 256), (3, 7, 4096), (8, 64, 1024), (4, 100, 8192), (7, 1000, 272), (2, 1536, 4096),
+                    # two tokens with long rows (up to 11264 codes), and just past that limit
+                    (2, 2048, 9232), (2, 4099, 11008), (2, 300, 11264), (2, 2048, 11280)]
 
 
 @pytest.mark.parametrize("rows_kernel", ["1", "0", None])

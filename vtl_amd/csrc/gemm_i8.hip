@@ -1512,7 +1512,7 @@ int launch_gemv(const GemmArgs &g, hipStream_t st)
     return check_launch("linear_gemv_kernel");
 }
 
-// A few tokens (2 <= M <= 8) against a weight matrix of rows up to 1024 * 32 / MR bytes.
+// A few tokens (2 <= M <= 8): rows of up to 11264 (2 tokens), 8192 (4) or 4096 (8) codes.
 template <int KV, int MR, bool DYNQ, bool F32OUT>
 int launch_gemv_rows_kv(const GemmArgs &g, hipStream_t st)
 {
@@ -1544,9 +1544,15 @@ int launch_gemv_rows_mr(const GemmArgs &g, hipStream_t st)
         return launch_gemv_rows_kv<2, MR, DYNQ, F32OUT>(g, st);
     if (kv <= 4)
         return launch_gemv_rows_kv<4, MR, DYNQ, F32OUT>(g, st);
-    if constexpr (MR <= 4)
-        return launch_gemv_rows_kv<8, MR, DYNQ, F32OUT>(g, st);
-    return VTL_HIP_ERR_UNSUPPORTED;  // not reached: 8 rows are routed here up to K = 4096
+    if constexpr (MR <= 4) {
+        if (kv <= 8)
+            return launch_gemv_rows_kv<8, MR, DYNQ, F32OUT>(g, st);
+    }
+    if constexpr (MR <= 2) {
+        if (kv <= 11)
+            return launch_gemv_rows_kv<11, MR, DYNQ, F32OUT>(g, st);
+    }
+    return VTL_HIP_ERR_UNSUPPORTED;  // not reached: see gemv_rows_applies
 }
 
 template <bool DYNQ, bool F32OUT>
@@ -1559,10 +1565,12 @@ int launch_gemv_rows(const GemmArgs &g, hipStream_t st)
     return launch_gemv_rows_mr<8, DYNQ, F32OUT>(g, st);
 }
 
-// The codes of the MR rows stay in registers: at most 32 pieces of 16 bytes per lane.
+// The codes of the MR rows stay in registers: at most 32 pieces of 16 bytes per lane (22 for two rows:
+// their weight rows are longer).
 inline bool gemv_rows_applies(const void *rows, const void *w, int M, int N, int K)
 {
-    return M >= 2 && M <= 8 && K % 16 == 0 && K >= 256 && K <= (M <= 4 ? 8192 : 4096) && aligned16(rows) &&
+    return M >= 2 && M <= 8 && K % 16 == 0 && K >= 256 && K <= (M <= 2 ? 11264 : (M <= 4 ? 8192 : 4096)) &&
+           aligned16(rows) &&
            aligned16(w) && !getenv("VTL_HIP_NO_GEMV");
 }
 
