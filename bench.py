@@ -380,6 +380,33 @@ def bench_copy_calibration(timer: Timer, steps: int, warmup: int):
             "kernel_us": dev_ms / steps * 1e3, "GB/s": gbps}
 
 
+def bench_mfma_only(timer: Timer):
+    """What the matrix cores alone sustain: the library's probe kernel runs nothing but the
+    int8 MFMA of the matmul kernels, once on constant operands and once on uniformly random
+    ones (the operand distribution of configs[2]), each for a few tens of milliseconds so
+    that the clock has settled.  The random-operand figure is the ceiling that the power
+    limit leaves to any int8 kernel on such data; the Linear's fraction of it is reported
+    next to its fraction of the nominal peak."""
+    rng = np.random.Generator(np.random.Philox(2))
+    sink = HipTensor.empty([4], np.int32)
+    out = {}
+    iters = 4000
+    ops = 1024.0 * 4 * 16 * iters * 65536.0
+    for label, host in (("constant_operands", np.full(32768, 1, np.int8)),
+                        ("uniform_random_operands", rng.integers(-127, 128, 32768, dtype=np.int8))):
+        buf = HipTensor.from_host(host)
+
+        def step():
+            capi.call("vtl_hip_probe_mfma_i8", buf.ptr, iters, sink.ptr)
+        for _ in range(4):
+            step()
+        _, dev_ms = timer.run(step, 8)
+        out[label] = {"TOP/s": ops / (dev_ms / 8 * 1e-3) / 1e12, "us_per_launch": dev_ms / 8 * 1e3}
+        buf.release()
+    sink.release()
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -388,7 +415,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=300)
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["all", "linear", "quant", "copy", "full", "other"], default="all")
+    ap.add_argument("--only", choices=["all", "linear", "quant", "copy", "full", "other", "mfma"], default="all")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 "
@@ -409,6 +436,9 @@ def main() -> int:
         return 0
     if args.only == "other":
         print(json.dumps({"other_configs": bench_other_configs(timer, args.steps, args.warmup)}))
+        return 0
+    if args.only == "mfma":
+        print(json.dumps({"mfma_only": bench_mfma_only(timer)}))
         return 0
 
     lin = bench_linear(timer, args.steps, args.warmup, cpu) if args.only in ("all", "linear") else None
@@ -441,6 +471,10 @@ def main() -> int:
     if qd:
         line["quantize"] = qd["quantize"]
         line["dequantize"] = qd["dequantize"]
+    if lin:
+        line["mfma_only"] = bench_mfma_only(timer)
+        line["roofline"]["frac_of_mfma_only_rate_on_these_operands"] = (
+            line["roofline"]["achieved"] / line["mfma_only"]["uniform_random_operands"]["TOP/s"])
     if args.only == "all":
         line["other_configs"] = bench_other_configs(timer, args.steps, args.warmup)
         line["full_precision"] = bench_full_precision(timer, args.steps, args.warmup)

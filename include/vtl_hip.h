@@ -151,6 +151,14 @@ int vtl_hip_linear_f32_dynquant(const float *X, const int8_t *Wq, const float *s
                                 const float *bias, float *Y, int M, int N, int K, int relu,
                                 void *workspace, size_t workspace_bytes);
 
+/* Measurement aid (no counterpart in the reference): runs nothing but the
+ * int8 MFMA of the matmul kernels - 1024 workgroups of 4 waves, each wave
+ * `iterations` times 16 instructions of 32x32x32 on operand registers loaded
+ * once from `operands` (32 KiB, 16-byte aligned, device) - so that a caller can
+ * time what the matrix cores sustain on given operand bits:
+ * ops = 1024 * 4 * 16 * iterations * 65536.  `sink` is one int32 on the device. */
+int vtl_hip_probe_mfma_i8(const int8_t *operands, int iterations, int32_t *sink);
+
 /* ---- f32 / f64 matmul with f64 accumulation ------------------------------ */
 
 /* C[M,N] = op(A) . op(B) with every product and sum in f64 and one rounding

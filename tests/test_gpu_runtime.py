@@ -167,3 +167,17 @@ def test_entry_points_capture_into_a_hip_graph(hip):
         hiprt.hipStreamDestroy(stream)
         for t in (X, W, SW, B, XQ, SX, Y):
             t.release()
+
+
+def test_mfma_probe_runs_and_leaves_its_sink_alone(hip):
+    """The measurement aid behind bench.py's `mfma_only` figures: launches, finishes, and
+    never writes its sink (the sums it keeps alive cannot reach the sentinel)."""
+    ops = HipTensor.from_host(np.random.default_rng(0).integers(-127, 128, 32768, dtype=np.int8))
+    sink = HipTensor.from_host(np.array([-7, 0, 0, 0], np.int32))
+    capi.call("vtl_hip_probe_mfma_i8", ops.ptr, 3, sink.ptr)
+    capi.call("vtl_hip_probe_mfma_i8", ops.ptr, 0, sink.ptr)
+    capi.call("vtl_hip_sync")
+    assert sink.cpu()[0] == -7
+    assert capi.status("vtl_hip_probe_mfma_i8", ops.ptr + 1, 3, sink.ptr) == capi.ERR_INVALID_ARG
+    ops.release()
+    sink.release()

@@ -1184,6 +1184,43 @@ __global__ __launch_bounds__(512) void linear_gemv_rows_kernel(const GemmArgs g)
 }
 
 
+// Measurement aid, not on the compute path: nothing but the MFMA of the tile
+// kernels, 16 independent 32x32 accumulators per wave fed from registers that
+// are loaded once (8 operand vectors per lane from `operands`, 32 KiB), four
+// waves on every SIMD of the chip.  What this loop sustains on given operand
+// bits is the ceiling of any int8 kernel on them: with constant operands the
+// nominal rate, with random ones whatever the power limit leaves.
+__global__ __launch_bounds__(256) void mfma_i8_probe_kernel(const int8_t *__restrict__ operands, int iterations,
+                                                            int32_t *sink)
+{
+    const v4i *in = reinterpret_cast<const v4i *>(operands) + threadIdx.x * 8;
+    v4i a[4], b[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        a[i] = in[i];
+        b[i] = in[4 + i];
+    }
+    v16i acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+            acc[i][r] = 0;
+    for (int it = 0; it < iterations; it++) {
+#pragma unroll
+        for (int i = 0; i < 16; i++)
+            acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i & 3], b[i >> 2], acc[i], 0, 0, 0);
+    }
+    int s = 0;
+#pragma unroll
+    for (int i = 0; i < 16; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+            s += acc[i][r];
+    if (s == 0x7fffffff)   // keeps the loop alive; practically never true
+        sink[0] = s;
+}
+
 // Any shape, any alignment: one output per thread.  Only used when K is not a
 // multiple of 16 or a pointer is not 16-byte aligned.
 template <bool F32OUT>
@@ -1679,6 +1716,14 @@ int check_gemm_args(const void *A, const void *Bt, const void *out, int M, int N
 }  // namespace
 
 extern "C" {
+
+int vtl_hip_probe_mfma_i8(const int8_t *operands, int iterations, int32_t *sink)
+{
+    if (!operands || !sink || iterations < 0 || !aligned16(operands))
+        return VTL_HIP_ERR_INVALID_ARG;
+    hipLaunchKernelGGL(mfma_i8_probe_kernel, dim3(1024), dim3(256), 0, current_stream(), operands, iterations, sink);
+    return check_launch("mfma_i8_probe_kernel");
+}
 
 int vtl_hip_gemm_i8_i32(const int8_t *A, const int8_t *Bt, int32_t *C, int M, int N, int K)
 {
