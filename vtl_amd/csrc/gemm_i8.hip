@@ -1464,7 +1464,7 @@ int launch_config(int idx, const GemmArgs &g, int splits, hipStream_t st)
 // plus, for split K, the extra launch and the pass over the partial sums.
 // The constants were fitted (random search, least mean log regret) to an
 // exhaustive timing sweep of every tile and split count over 55 shapes (mean
-// regret 1 %, worst 10 %).
+// regret 0.6 %, worst 10 %).
 void choose_config(int M, int N, int K, int &best_idx, int &best_splits)
 {
     const int kt_all = (K + 127) / 128;
@@ -1476,6 +1476,12 @@ void choose_config(int M, int N, int K, int &best_idx, int &best_splits)
         if (i > 0 && kTileConfigs[i - 1].bm >= M && c.bm > kTileConfigs[i - 1].bm)
             break;  // a taller tile would only add padding rows
         const int64_t tiles = (int64_t)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
+        // More than one round of 256x256 tiles with a short K: each round pays the long fill and
+        // the 256 KiB store of a tile that owns its compute unit, while two 128x128 tiles per
+        // compute unit overlap theirs (8192x8192x1024: 97 against 104 us, 6144x6144x2048: 90
+        // against 98 us).
+        if (c.bm == 256 && K <= 2048 && tiles > 256)
+            continue;
         for (int s = 1; s <= 16; s *= 2) {
             if (s > 1 && kt_all / s < 4)
                 break;
