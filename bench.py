@@ -381,12 +381,20 @@ def bench_copy_calibration(timer: Timer, steps: int, warmup: int):
 
 
 def bench_mfma_only(timer: Timer):
-    """What the matrix cores alone sustain: the library's probe kernel runs nothing but the
+    """What the matrix cores alone sustain: a probe kernel (a small library of its own, built
+    beside the product library and loaded only here) runs nothing but the
     int8 MFMA of the matmul kernels, once on constant operands and once on uniformly random
     ones (the operand distribution of configs[2]), each for a few tens of milliseconds so
     that the clock has settled.  The random-operand figure is the ceiling that the power
     limit leaves to any int8 kernel on such data; the Linear's fraction of it is reported
     next to its fraction of the nominal peak."""
+    from vtl_amd import build as vb
+    if not os.path.exists(vb.BENCH_PROBE_PATH):
+        vb.build_lib()
+    probe = C.CDLL(vb.BENCH_PROBE_PATH).vtl_bench_probe_mfma_i8
+    probe.restype, probe.argtypes = C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
+    stream = C.c_void_p()
+    capi.call("vtl_hip_get_stream", C.byref(stream))
     rng = np.random.Generator(np.random.Philox(2))
     sink = HipTensor.empty([4], np.int32)
     out = {}
@@ -397,7 +405,8 @@ def bench_mfma_only(timer: Timer):
         buf = HipTensor.from_host(host)
 
         def step():
-            capi.call("vtl_hip_probe_mfma_i8", buf.ptr, iters, sink.ptr)
+            if probe(buf.ptr, iters, sink.ptr, stream) != 0:
+                raise RuntimeError("vtl_bench_probe_mfma_i8 failed")
         for _ in range(4):
             step()
         _, dev_ms = timer.run(step, 8)

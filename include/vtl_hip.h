@@ -25,7 +25,17 @@
  *     LinearLayer, `[out_features, in_features]` (nn/layers/linear.v:10-16),
  *     never as a transposed view;
  *   - one host thread per device; the library keeps no pointers to caller
- *     memory after a call returns.
+ *     memory after a call returns;
+ *   - a few entry points stage data in scratch memory the library owns (the
+ *     K-split partial sums of the matmuls, vtl_hip_linear_i8_requant,
+ *     vtl_hip_linear_f32_dynquant with workspace == NULL, int8 operands that
+ *     need repacking).  There is one such buffer per purpose and device,
+ *     shared by every stream: calls that use it must not overlap on a device,
+ *     i.e. issue them on one stream (or order the streams yourself).  The
+ *     buffers grow on demand, which waits for the whole device; while the
+ *     current stream is being captured into a graph a call that would have to
+ *     grow one returns VTL_HIP_ERR_UNSUPPORTED instead (run it once before
+ *     capturing).
  */
 #ifndef VTL_HIP_H
 #define VTL_HIP_H
@@ -151,14 +161,6 @@ int vtl_hip_linear_f32_dynquant(const float *X, const int8_t *Wq, const float *s
                                 const float *bias, float *Y, int M, int N, int K, int relu,
                                 void *workspace, size_t workspace_bytes);
 
-/* Measurement aid (no counterpart in the reference): runs nothing but the
- * int8 MFMA of the matmul kernels - 1024 workgroups of 4 waves, each wave
- * `iterations` times 16 instructions of 32x32x32 on operand registers loaded
- * once from `operands` (32 KiB, 16-byte aligned, device) - so that a caller can
- * time what the matrix cores sustain on given operand bits:
- * ops = 1024 * 4 * 16 * iterations * 65536.  `sink` is one int32 on the device. */
-int vtl_hip_probe_mfma_i8(const int8_t *operands, int iterations, int32_t *sink);
-
 /* ---- f32 / f64 matmul with f64 accumulation ------------------------------ */
 
 /* C[M,N] = op(A) . op(B) with every product and sum in f64 and one rounding
@@ -222,6 +224,10 @@ const char *vtl_hip_strerror(int status);
 /* Text of the last HIP runtime error seen by this thread ("" if none). */
 const char *vtl_hip_last_error(void);
 const char *vtl_hip_version(void);
+/* The library reads its tuning switches (environment variables VTL_HIP_*, used
+ * by tests and tuning runs only) once, at the first call that looks at them;
+ * this reads them again. */
+int vtl_hip_reload_env(void);
 
 #ifdef __cplusplus
 }

@@ -72,8 +72,6 @@ def test_bad_arguments_return_status_not_abort():
     assert S("vtl_hip_linear_i8_requant", one, one, 1, one, one, 1, None, 0, one, one, None, 0, 4, 16) == capi.OK
     assert S("vtl_hip_linear_f32_dynquant", one, one, one, None, one, 4, 4, 16, 0, C.c_void_p(20), 4096) == E   # misaligned
     assert S("vtl_hip_linear_f32_dynquant", one, one, one, None, one, 4, 4, 16, 0, one, 8) == E
-    assert S("vtl_hip_probe_mfma_i8", None, 1, one) == E
-    assert S("vtl_hip_probe_mfma_i8", one, -1, one) == E
     assert S("vtl_hip_relu_f32", None, 4) == E
     assert S("vtl_hip_event_record", None) == E
     # empty problems succeed without touching the device

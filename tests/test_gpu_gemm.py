@@ -171,6 +171,9 @@ def test_square_gemm_config_full_size(hip):
 ROUTED_SHAPES = [(1, 2048, 256), (1, 5, 256), (1, 4099, 4080), (1, 9000, 5120), (1, 300, 8192), (1, 2048, 8448),
                  (1, 9000, 9232), (1, 4097, 11264), (1, 8192, 14336), (1, 100, 14352), (1, 3000, 16384),
                  (1, 262200, 256),      # more rows than the matrix-vector kernel deals out
+                 # rows longer than 6144 codes run on half as many waves: 64 rows per wave is the
+                 # most a wave can park (131072 rows), one row more leaves the matrix-vector kernel
+                 (1, 131072, 6160), (1, 131073, 6160), (1, 152064, 8192),
 
                  (3, 2050, 256), (8, 2048, 4096), (9, 2048, 768), (16, 2047, 1280),
                  (17, 2077, 1280), (32, 4096, 512), (31, 14336, 256), (5, 3001, 4096),
@@ -184,13 +187,13 @@ SMALL_SHAPES = [(64, 256, 784), (1, 1, 16), (2, 3, 16), (33, 65, 48), (64, 64, 2
 
 @pytest.mark.parametrize("small", ["0", "1", None])
 @pytest.mark.parametrize("mnk", SMALL_SHAPES)
-def test_small_product_kernel_and_its_alternatives(hip, mnk, small, monkeypatch):
+def test_small_product_kernel_and_its_alternatives(hip, mnk, small, knobs):
     """VTL_HIP_GEMM_SMALL=1 forces the small-product kernel, 0 the tile kernels the
     same shapes used before it existed, unset the library's own choice."""
     if small is None:
-        monkeypatch.delenv("VTL_HIP_GEMM_SMALL", raising=False)
+        knobs.delenv("VTL_HIP_GEMM_SMALL", raising=False)
     else:
-        monkeypatch.setenv("VTL_HIP_GEMM_SMALL", small)
+        knobs.setenv("VTL_HIP_GEMM_SMALL", small)
     m, n, k = mnk
     a, bt, sa, sb, bias = workloads.square_int8_gemm(m, n, k, seed=m * 17 + n * 5 + k)
     ref = oracle.gemm_i8_i32(a, bt, threads=CPU_THREADS)
@@ -237,13 +240,13 @@ FEW_TOKEN_SHAPES = [(2, 2048, 256), (2, 3001, 1008), (2, 2050, 2048), (2, 2048, 
 
 @pytest.mark.parametrize("rows_kernel", ["1", "0", None])
 @pytest.mark.parametrize("mnk", FEW_TOKEN_SHAPES)
-def test_few_token_kernel_and_its_alternatives(hip, mnk, rows_kernel, monkeypatch):
+def test_few_token_kernel_and_its_alternatives(hip, mnk, rows_kernel, knobs):
     """VTL_HIP_GEMV_ROWS=1 forces the few-token kernel wherever it applies, 0 keeps it
     off, unset is the library's own choice: int32 sums and f32 epilogue are those of the oracle."""
     if rows_kernel is None:
-        monkeypatch.delenv("VTL_HIP_GEMV_ROWS", raising=False)
+        knobs.delenv("VTL_HIP_GEMV_ROWS", raising=False)
     else:
-        monkeypatch.setenv("VTL_HIP_GEMV_ROWS", rows_kernel)
+        knobs.setenv("VTL_HIP_GEMV_ROWS", rows_kernel)
     m, n, k = mnk
     a, bt, sa, sb, bias = workloads.square_int8_gemm(m, n, k, seed=m * 31 + n * 3 + k)
     ref = oracle.gemm_i8_i32(a, bt, threads=CPU_THREADS)
@@ -261,7 +264,7 @@ def test_few_token_kernel_and_its_alternatives(hip, mnk, rows_kernel, monkeypatc
 
 
 @pytest.mark.parametrize("k", [2432, 2448, 80])   # 19 K steps of 128; the same plus a 16-byte tail; one partial step
-def test_forced_split_k_is_exact(hip, monkeypatch, k):
+def test_forced_split_k_is_exact(hip, knobs, k):
     """Every tile configuration with 1, 2, 3 and 8 K ranges gives the same int32 result
     (uneven ranges for every split count)."""
     m, n = 96, 384
@@ -271,11 +274,11 @@ def test_forced_split_k_is_exact(hip, monkeypatch, k):
     A, B, dsa, dsb, dbias = dev(a), dev(bt), dev(sa), dev(sb), dev(bias)
     for idx in range(6):
         for splits in (1, 2, 3, 8):
-            monkeypatch.setenv("VTL_HIP_GEMM_CONFIG", f"{idx},{splits}")
+            knobs.setenv("VTL_HIP_GEMM_CONFIG", f"{idx},{splits}")
             assert np.array_equal(_gemm(a, bt), ref), (idx, splits)
             y = linear_i8_hip(A, dsa, B, dsb, dbias)
             assert np.array_equal(y.cpu(), want), (idx, splits)
             y.release()
-    monkeypatch.delenv("VTL_HIP_GEMM_CONFIG")
+    knobs.delenv("VTL_HIP_GEMM_CONFIG")
     for h in (A, B, dsa, dsb, dbias):
         h.release()

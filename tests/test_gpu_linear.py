@@ -74,7 +74,7 @@ REQUANT_SHAPES = [(256, 1024, 4096), (256, 4096, 11008), (256, 11008, 4096), (10
 
 
 @pytest.mark.parametrize("mnk", REQUANT_SHAPES)
-def test_requantizing_linear_equals_linear_then_row_quantize(hip, mnk, monkeypatch):
+def test_requantizing_linear_equals_linear_then_row_quantize(hip, mnk, knobs):
     """vtl_hip_linear_i8_requant gives the codes, scales and (when asked for) f32 rows of
     vtl_hip_linear_i8_f32 followed by the per-row quantizer, and of the oracle."""
     m, n, k = mnk
@@ -92,9 +92,9 @@ def test_requantizing_linear_equals_linear_then_row_quantize(hip, mnk, monkeypat
         assert np.array_equal(yq.cpu(), q_ref)
         yq2, sy2 = linear_i8_requant_hip(A, SA, W, SW, b_dev, relu=relu)       # no f32 rows wanted
         assert np.array_equal(yq2.cpu(), q_ref) and np.array_equal(sy2.cpu(), s_ref)
-        monkeypatch.setenv("VTL_HIP_NO_FUSED_REQUANT", "1")                    # linear, then row quantizer
+        knobs.setenv("VTL_HIP_NO_FUSED_REQUANT", "1")                    # linear, then row quantizer
         yq3, sy3 = linear_i8_requant_hip(A, SA, W, SW, b_dev, relu=relu)
-        monkeypatch.delenv("VTL_HIP_NO_FUSED_REQUANT")
+        knobs.delenv("VTL_HIP_NO_FUSED_REQUANT")
         assert np.array_equal(yq3.cpu(), q_ref) and np.array_equal(sy3.cpu(), s_ref)
         for h in (yq, sy, y, yq2, sy2, yq3, sy3):
             h.release()
@@ -181,7 +181,7 @@ def test_session_reuses_buffers_on_second_forward(hip):
                                  (5, 2048, 512), (8, 2050, 1024), (7, 9000, 1008), (6, 2048, 16 * 17),
                                  (8, 70001, 256), (2, 1, 256), (3, 7, 2048), (8, 64, 1024), (4, 100, 272),
                                  (2, 1536, 4096)])
-def test_few_token_fused_decode_equals_two_launch_path(hip, mnk, monkeypatch):
+def test_few_token_fused_decode_equals_two_launch_path(hip, mnk, knobs):
     """2 to 8 tokens with short rows take the few-token kernel whose workgroups quantize the
     rows themselves (forced here for every size it is built for); it must give the bits of
     the quantize-then-linear path and of the oracle, special values included."""
@@ -197,15 +197,15 @@ def test_few_token_fused_decode_equals_two_launch_path(hip, mnk, monkeypatch):
     bias = rng.standard_normal(n).astype(np.float32)
     X, W, SW, B = dev(x), dev(w), dev(sw), dev(bias)
     want = oracle.linear_f32_dynquant(x, w, sw, bias, relu=True, threads=CPU_THREADS)
-    monkeypatch.setenv("VTL_HIP_GEMV_ROWS", "1")
+    knobs.setenv("VTL_HIP_GEMV_ROWS", "1")
     fused = linear_f32_dynquant_hip(X, W, SW, B, relu=True).cpu()
-    monkeypatch.setenv("VTL_HIP_NO_FUSED_DECODE", "1")
+    knobs.setenv("VTL_HIP_NO_FUSED_DECODE", "1")
     plain = linear_f32_dynquant_hip(X, W, SW, B, relu=True).cpu()
-    monkeypatch.delenv("VTL_HIP_NO_FUSED_DECODE")
-    monkeypatch.delenv("VTL_HIP_GEMV_ROWS")
+    knobs.delenv("VTL_HIP_NO_FUSED_DECODE")
+    knobs.delenv("VTL_HIP_GEMV_ROWS")
     auto = linear_f32_dynquant_hip(X, W, SW, B, relu=True).cpu()
     assert np.array_equal(fused, want) and np.array_equal(plain, want) and np.array_equal(auto, want)
-    monkeypatch.setenv("VTL_HIP_GEMV_ROWS", "1")
+    knobs.setenv("VTL_HIP_GEMV_ROWS", "1")
     for special in (np.nan, np.inf, -np.inf):
         xs = x.copy()
         xs[0, 7] = special
@@ -221,8 +221,10 @@ def test_few_token_fused_decode_equals_two_launch_path(hip, mnk, monkeypatch):
 
 @pytest.mark.parametrize("nk", [(2048, 256), (2050, 512), (3001, 4096), (2077, 1280), (1, 16), (7, 48), (300, 784),
                                 (14336, 4080), (4097, 5120), (2048, 8192), (1000, 7168), (2050, 8208),
-                                (64, 11008), (2050, 9232), (4096, 11008), (300, 11280), (1000, 14336), (70, 14352)])
-def test_single_token_fused_decode_equals_two_launch_path(hip, nk, monkeypatch):
+                                (64, 11008), (2050, 9232), (4096, 11008), (300, 11280), (1000, 14336), (70, 14352),
+                                # long rows and more weight rows than 64 per wave of the halved grid
+                                (131072, 6160), (131073, 6160), (152064, 8192)])
+def test_single_token_fused_decode_equals_two_launch_path(hip, nk, knobs):
     """M = 1 takes the matrix-vector kernel that quantizes the token itself (rows of
     up to 14336 codes, any multiple of 16; longer rows take two launches); it must
     give the bits of the quantize-then-linear path and of the oracle."""
@@ -236,12 +238,12 @@ def test_single_token_fused_decode_equals_two_launch_path(hip, nk, monkeypatch):
     X, W, SW, B = dev(x), dev(w), dev(sw), dev(bias)
     want = oracle.linear_f32_dynquant(x, w, sw, bias, relu=True, threads=CPU_THREADS)
     fused = linear_f32_dynquant_hip(X, W, SW, B, relu=True).cpu()
-    monkeypatch.setenv("VTL_HIP_NO_FUSED_DECODE", "1")
+    knobs.setenv("VTL_HIP_NO_FUSED_DECODE", "1")
     plain = linear_f32_dynquant_hip(X, W, SW, B, relu=True).cpu()
     assert np.array_equal(fused, want) and np.array_equal(plain, want)
     # degenerate token: all zeros -> scale 0 -> output is the bias (ReLU applied)
     Z = dev(np.zeros((1, k), np.float32))
-    monkeypatch.delenv("VTL_HIP_NO_FUSED_DECODE")
+    knobs.delenv("VTL_HIP_NO_FUSED_DECODE")
     got = linear_f32_dynquant_hip(Z, W, SW, B, relu=False).cpu()
     assert np.array_equal(got, oracle.linear_f32_dynquant(np.zeros((1, k), np.float32), w, sw, bias))
     # NaN elements are ignored by the absmax and quantize to 0; an infinite element makes the

@@ -67,7 +67,7 @@ def test_matmul_shapes_and_layouts(hip, dt, ta, tb):
 
 
 @pytest.mark.parametrize("dt", [np.float32, np.float64])
-def test_split_k_paths(hip, dt, monkeypatch):
+def test_split_k_paths(hip, dt, knobs):
     """Few output tiles and a long K slice K over the grid; forced slice counts cover
     ragged K, edge tiles and the unsplit fallback."""
     rng = np.random.default_rng(27)
@@ -76,9 +76,9 @@ def test_split_k_paths(hip, dt, monkeypatch):
              (33, 65, 777, False, False, "16"), (64, 128, 96, False, True, "4")]
     for (M, N, K, ta, tb, force) in cases:
         if force is None:
-            monkeypatch.delenv("VTL_HIP_MATMUL_SPLITS", raising=False)
+            knobs.delenv("VTL_HIP_MATMUL_SPLITS", raising=False)
         else:
-            monkeypatch.setenv("VTL_HIP_MATMUL_SPLITS", force)
+            knobs.setenv("VTL_HIP_MATMUL_SPLITS", force)
         A = rng.standard_normal((K, M) if ta else (M, K)).astype(dt)
         B = rng.standard_normal((N, K) if tb else (K, N)).astype(dt)
         print("split-K", dt.__name__, M, N, K, ta, tb, force, flush=True)
@@ -91,7 +91,7 @@ def test_split_k_paths(hip, dt, monkeypatch):
         exact = (Ai.T if ta else Ai).astype(np.float64) @ (Bi.T if tb else Bi).astype(np.float64)
         assert np.array_equal(run_matmul(Ai, Bi, ta, tb), exact.astype(dt))
     # the Linear form keeps bias and ReLU after the sliced sum
-    monkeypatch.delenv("VTL_HIP_MATMUL_SPLITS", raising=False)
+    knobs.delenv("VTL_HIP_MATMUL_SPLITS", raising=False)
     x = rng.standard_normal((128, 4096)).astype(dt)
     w = (rng.standard_normal((256, 4096)) * 0.05).astype(dt)
     b = rng.standard_normal(256).astype(dt)
@@ -105,10 +105,10 @@ def test_split_k_paths(hip, dt, monkeypatch):
 
 
 @pytest.mark.parametrize("tile", ["64", "128"])
-def test_forced_tile_sizes(hip, tile, monkeypatch):
+def test_forced_tile_sizes(hip, tile, knobs):
     """VTL_HIP_MATMUL_TILE forces the 64x64 or the 128x128 tile kernel: whole and ragged
     tiles, all four layouts, both give the oracle's result (integers bit for bit)."""
-    monkeypatch.setenv("VTL_HIP_MATMUL_TILE", tile)
+    knobs.setenv("VTL_HIP_MATMUL_TILE", tile)
     rng = np.random.default_rng(int(tile))
     for (M, N, K, ta, tb) in [(256, 384, 128, False, True), (300, 200, 96, True, False), (129, 65, 260, True, True),
                               (1, 1, 1, False, False), (640, 512, 64, False, False)]:

@@ -2,6 +2,7 @@
 (the calls HipStorage makes where CudaStorage calls cudaMalloc / cudaMemcpy /
 cudaFree, storage/cuda_d_cuda.v:32-102)."""
 import ctypes as C
+import os
 
 import numpy as np
 import pytest
@@ -174,10 +175,14 @@ def test_mfma_probe_runs_and_leaves_its_sink_alone(hip):
     never writes its sink (the sums it keeps alive cannot reach the sentinel)."""
     ops = HipTensor.from_host(np.random.default_rng(0).integers(-127, 128, 32768, dtype=np.int8))
     sink = HipTensor.from_host(np.array([-7, 0, 0, 0], np.int32))
-    capi.call("vtl_hip_probe_mfma_i8", ops.ptr, 3, sink.ptr)
-    capi.call("vtl_hip_probe_mfma_i8", ops.ptr, 0, sink.ptr)
+    from vtl_amd import build as vb
+    assert os.path.exists(vb.BENCH_PROBE_PATH), "libvtlbenchprobe.so is not built"
+    probe = C.CDLL(vb.BENCH_PROBE_PATH).vtl_bench_probe_mfma_i8
+    probe.restype, probe.argtypes = C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
+    assert probe(ops.ptr, 3, sink.ptr, None) == 0
+    assert probe(ops.ptr, 0, sink.ptr, None) == 0
     capi.call("vtl_hip_sync")
     assert sink.cpu()[0] == -7
-    assert capi.status("vtl_hip_probe_mfma_i8", ops.ptr + 1, 3, sink.ptr) == capi.ERR_INVALID_ARG
+    assert probe(ops.ptr + 1, 3, sink.ptr, None) == 1
     ops.release()
     sink.release()

@@ -32,6 +32,27 @@ def test_tensor_encoding_round_trip_and_errors():
         ser.decode_tensor(ser.encode_tensor(np.zeros((2, 3), np.float32)), [3, 2])
 
 
+def test_layer_definitions_known_answer(tmp_path):
+    """The LayerDef list a reference Sequential (input -> linear -> relu -> linear) writes:
+    nn/models/serialization.v:108-137 with sequential_info.v:43-60 (the input layer is layer 0,
+    in_shape empty; then each layer's in_shape is the output shape of the one before)."""
+    from vtl_amd import QuantLinearLayer
+    l1 = QuantLinearLayer(np.zeros((24, 48), np.float32))
+    l2 = QuantLinearLayer(np.zeros((8, 24), np.float32))
+    path = str(tmp_path / "defs.json")
+    ser.save_model(path, [l1, "relu", l2], [48], with_quantized=False)
+    text = open(path).read()
+    model = json.loads(text)
+    assert model["layers"] == [
+        {"layer_type": "InputLayer", "in_shape": [], "config": {"shape_0": 48}},
+        {"layer_type": "LinearLayer", "in_shape": [48], "config": {"in_features": 48, "out_features": 24}},
+        {"layer_type": "ReLULayer", "in_shape": [24], "config": {}},
+        {"layer_type": "LinearLayer", "in_shape": [24], "config": {"in_features": 24, "out_features": 8}}]
+    assert [list(d["weights"]) for d in model["layer_data"]] == [[], ["weight", "bias"], [], ["weight", "bias"]]
+    # key order of the Linear config as the reference inserts it
+    assert text.index('"in_features"') < text.index('"out_features"')
+
+
 @pytest.mark.gpu
 def test_model_file_round_trip_with_quantized_weights(hip, tmp_path):
     import oracle
@@ -42,9 +63,10 @@ def test_model_file_round_trip_with_quantized_weights(hip, tmp_path):
     path = str(tmp_path / "model.json")
     ser.save_model(path, [l1, "relu", l2], [48], epoch=3, loss=0.25)
     model = json.load(open(path))
-    assert model["version"] == "1.0" and [d["layer_type"] for d in model["layers"]] == ["LinearLayer", "ReLULayer", "LinearLayer"]
-    assert model["layers"][0]["config"] == {"out_features": 24, "in_features": 48}
-    assert set(model["layer_data"][0]["weights"]) == {"weight", "bias", "weight_q", "weight_scale"}
+    assert model["version"] == "1.0" and [d["layer_type"] for d in model["layers"]] == ["InputLayer", "LinearLayer", "ReLULayer", "LinearLayer"]
+    assert model["layers"][0]["in_shape"] == [] and model["layers"][1]["in_shape"] == [48]
+    assert model["layers"][1]["config"] == {"out_features": 24, "in_features": 48}
+    assert set(model["layer_data"][1]["weights"]) == {"weight", "bias", "weight_q", "weight_scale"}
     loaded = ser.load_linear_layers(path, PER_CHANNEL)
     assert len(loaded) == 2
     x = rng.standard_normal((5, 48)).astype(np.float32)
@@ -59,7 +81,7 @@ def test_model_file_round_trip_with_quantized_weights(hip, tmp_path):
     assert np.array_equal(h, l1.forward(x))
     # a file written without the extra keys is an ordinary reference model file
     ser.save_model(path, [l1], [48], with_quantized=False)
-    assert set(json.load(open(path))["layer_data"][0]["weights"]) == {"weight", "bias"}
+    assert set(json.load(open(path))["layer_data"][1]["weights"]) == {"weight", "bias"}
     assert ser.load_linear_layers(path)[0][1] is None
     for l in (l1, l2, loaded[0][0], loaded[1][0]):
         l.release()

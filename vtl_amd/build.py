@@ -11,6 +11,8 @@ REPO_ROOT = os.path.dirname(PKG_DIR)
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libvtlhip.so")
 OBJ_DIR = os.path.join(PKG_DIR, "_build")
+# bench.py's measurement aid (an MFMA-only loop): a library of its own, no part of the product
+BENCH_PROBE_PATH = os.path.join(PKG_DIR, "libvtlbenchprobe.so")
 SOURCES = ["runtime.hip", "quant.hip", "gemm_i8.hip", "matmul_f64acc.hip", "tensor_ops.hip"]
 
 HIPCC_FLAGS = [
@@ -66,8 +68,14 @@ def build_lib(verbose: bool = False, extra_flags: list[str] | None = None) -> st
         _run([hipcc(), *HIPCC_FLAGS, *SOURCE_FLAGS.get(src, []), *(extra_flags or []), *includes,
               "-c", os.path.join(CSRC, src), "-o", objects[i]], verbose)
 
-    with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as pool:
+    def compile_probe() -> None:
+        _run([hipcc(), "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+              os.path.join(CSRC, "bench_probe.hip"), "-o", BENCH_PROBE_PATH], verbose)
+
+    with ThreadPoolExecutor(max_workers=min(4, len(SOURCES) + 1)) as pool:
+        probe = pool.submit(compile_probe)
         list(pool.map(compile_one, range(len(SOURCES))))
+        probe.result()
     _run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *objects, "-o", LIB_PATH], verbose)
     return LIB_PATH
 

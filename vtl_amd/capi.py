@@ -49,7 +49,6 @@ SIGNATURES = {
     "vtl_hip_linear_i8_requant": (_ci, [_vp, _vp, _ci, _vp, _vp, _ci, _vp, _ci, _vp, _vp, _vp, _ci, _ci, _ci]),
     "vtl_hip_linear_f32_dynquant_workspace": (_sz, [_ci, _ci]),
     "vtl_hip_linear_f32_dynquant": (_ci, [_vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp, _sz]),
-    "vtl_hip_probe_mfma_i8": (_ci, [_vp, _ci, _vp]),
     "vtl_hip_matmul_f32": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci]),
     "vtl_hip_matmul_f64": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci]),
     "vtl_hip_linear_f32": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci]),
@@ -67,6 +66,7 @@ SIGNATURES = {
     "vtl_hip_strerror": (C.c_char_p, [_ci]),
     "vtl_hip_last_error": (C.c_char_p, []),
     "vtl_hip_version": (C.c_char_p, []),
+    "vtl_hip_reload_env": (_ci, []),
 }
 
 

@@ -29,6 +29,26 @@ bool launch_copy(void *dst, const void *src, size_t bytes, hipStream_t st);
 // current stream may use a slot until the next call that asks for it; nullptr
 // when the allocation fails.
 void *library_workspace(size_t bytes, int slot = 0);
+// Why the last library_workspace() call of this thread returned nullptr
+// (VTL_HIP_ERR_OUT_OF_MEMORY, or VTL_HIP_ERR_UNSUPPORTED when the buffer would
+// have to grow during a stream capture).
+int workspace_status();
+
+// Tuning and test switches, taken from the environment once (first use) and
+// again only when vtl_hip_reload_env() is called: the dispatch path of a launch
+// reads this struct, never the environment.
+struct Tuning {
+    bool no_gemv = false;           // VTL_HIP_NO_GEMV: keep M <= 8 off the matrix-vector kernels
+    int gemv_rows = -1;             // VTL_HIP_GEMV_ROWS: 1 / 0 force the few-token kernel on / off
+    int gemm_small = -1;            // VTL_HIP_GEMM_SMALL: 1 / 0 force the small-product kernel on / off
+    int gemm_config = -1;           // VTL_HIP_GEMM_CONFIG "<tile index>,<splits>"
+    int gemm_splits = 1;
+    bool no_fused_requant = false;  // VTL_HIP_NO_FUSED_REQUANT: linear, then the row quantizer
+    bool no_fused_decode = false;   // VTL_HIP_NO_FUSED_DECODE: quantizer launch in front of the linear
+    int matmul_tile = 0;            // VTL_HIP_MATMUL_TILE: 128 / 64 force the f64-accumulating tile
+    int matmul_splits = -1;         // VTL_HIP_MATMUL_SPLITS: K ranges of the f64-accumulating matmul
+};
+const Tuning &tuning();
 
 constexpr int kWave = 64;
 

@@ -1184,43 +1184,6 @@ __global__ __launch_bounds__(512) void linear_gemv_rows_kernel(const GemmArgs g)
 }
 
 
-// Measurement aid, not on the compute path: nothing but the MFMA of the tile
-// kernels, 16 independent 32x32 accumulators per wave fed from registers that
-// are loaded once (8 operand vectors per lane from `operands`, 32 KiB), four
-// waves on every SIMD of the chip.  What this loop sustains on given operand
-// bits is the ceiling of any int8 kernel on them: with constant operands the
-// nominal rate, with random ones whatever the power limit leaves.
-__global__ __launch_bounds__(256) void mfma_i8_probe_kernel(const int8_t *__restrict__ operands, int iterations,
-                                                            int32_t *sink)
-{
-    const v4i *in = reinterpret_cast<const v4i *>(operands) + threadIdx.x * 8;
-    v4i a[4], b[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        a[i] = in[i];
-        b[i] = in[4 + i];
-    }
-    v16i acc[16];
-#pragma unroll
-    for (int i = 0; i < 16; i++)
-#pragma unroll
-        for (int r = 0; r < 16; r++)
-            acc[i][r] = 0;
-    for (int it = 0; it < iterations; it++) {
-#pragma unroll
-        for (int i = 0; i < 16; i++)
-            acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i & 3], b[i >> 2], acc[i], 0, 0, 0);
-    }
-    int s = 0;
-#pragma unroll
-    for (int i = 0; i < 16; i++)
-#pragma unroll
-        for (int r = 0; r < 16; r++)
-            s += acc[i][r];
-    if (s == 0x7fffffff)   // keeps the loop alive; practically never true
-        sink[0] = s;
-}
-
 // Any shape, any alignment: one output per thread.  Only used when K is not a
 // multiple of 16 or a pointer is not 16-byte aligned.
 template <bool F32OUT>
@@ -1384,7 +1347,7 @@ int launch_dma(GemmArgs g, int splits, hipStream_t st)
         g.partials = static_cast<int32_t *>(
             vtlhip::library_workspace((size_t)splits * (size_t)g.M * (size_t)g.N * sizeof(int32_t)));
         if (!g.partials)
-            return VTL_HIP_ERR_OUT_OF_MEMORY;
+            return vtlhip::workspace_status();
     }
     static PerDevice<bool> done_flags[6];
     bool *done[6] = {&done_flags[0].get(), &done_flags[1].get(), &done_flags[2].get(),
@@ -1526,16 +1489,21 @@ int launch_skinny(const GemmArgs &g, hipStream_t st)
     return launch_skinny_cfg<2, 2, 4, F32OUT>(g, st);
 }
 
+// Waves of the single-token kernel's grid: no more than the chip holds at once, sixteen per
+// compute unit up to 6144 codes a row, eight beyond (the codes and three weight rows of a wave
+// take 150 to 250 registers then).
+inline int gemv_max_waves(int K) { return K <= 6144 ? 4096 : 2048; }
+
 // Single-token linear (M = 1, K % 16 == 0, K <= 14336, operands 16-byte aligned).
 template <bool DYNQ, bool F32OUT>
 int launch_gemv(const GemmArgs &g, hipStream_t st)
 {
     constexpr int NWAVE = 8;
-    // every wave the same number of rows, and no more waves than the chip holds at once: sixteen
-    // per compute unit up to 6144 codes a row, eight beyond (the codes and three weight rows of a
-    // wave take 150 to 250 registers then)
-    const int max_waves = g.K <= 6144 ? 4096 : 2048;
+    // every wave the same number of rows
+    const int max_waves = gemv_max_waves(g.K);
     const int rows_per_wave = (g.N + max_waves - 1) / max_waves;
+    if (rows_per_wave > 64)   // more rows than a wave has lanes to park their sums in
+        return VTL_HIP_ERR_UNSUPPORTED;
     const int64_t waves = (g.N + rows_per_wave - 1) / rows_per_wave;
     const dim3 grid((unsigned)((waves + NWAVE - 1) / NWAVE)), block(64 * NWAVE);
     switch ((g.K + 1023) / 1024) {
@@ -1614,7 +1582,7 @@ inline bool gemv_rows_applies(const void *rows, const void *w, int M, int N, int
 {
     return M >= 2 && M <= 8 && K % 16 == 0 && K >= 256 && K <= (M <= 2 ? 11264 : (M <= 4 ? 8192 : 4096)) &&
            aligned16(rows) &&
-           aligned16(w) && !getenv("VTL_HIP_NO_GEMV");
+           aligned16(w) && !tuning().no_gemv;
 }
 
 // Where the few-token kernel beats the MFMA weight-streaming kernel (measured, N = 64 ... 28672,
@@ -1622,8 +1590,8 @@ inline bool gemv_rows_applies(const void *rows, const void *w, int M, int N, int
 // LDS staging and a lower fixed cost.  Shapes the other kernel cannot take (K % 256 != 0) come here.
 inline bool gemv_rows_faster(int M, int N, int K)
 {
-    if (const char *force = getenv("VTL_HIP_GEMV_ROWS"))   // "1" / "0" force the choice (tests, tuning)
-        return atoi(force) != 0;
+    if (tuning().gemv_rows >= 0)   // 1 / 0 force the choice (tests, tuning)
+        return tuning().gemv_rows != 0;
     if (M <= 2 || K % 256 != 0 || N < 2048)   // few weight rows: never slower, 1.8x faster from K = 4096 on
         return true;
     if (M <= 4)
@@ -1637,15 +1605,16 @@ inline bool gemv_rows_faster(int M, int N, int K)
 inline bool gemv_rows_fused_quant_faster(int M, int N, int K)
 {
     const int mr = M <= 2 ? 2 : (M <= 4 ? 4 : 8);
-    if (const char *force = getenv("VTL_HIP_GEMV_ROWS"))   // only the instantiated sizes can be forced
-        return atoi(force) != 0 && (int64_t)mr * ((K + 1023) / 1024) <= 8;
+    if (tuning().gemv_rows >= 0)   // only the instantiated sizes can be forced
+        return tuning().gemv_rows != 0 && (int64_t)mr * ((K + 1023) / 1024) <= 8;
     return (int64_t)mr * K <= 8192 && (mr < 8 || (int64_t)N * K <= (int64_t)4 << 20);
 }
 
-// N <= 64 * 4096: a wave parks one sum per lane.
+// A wave parks one sum per lane, so it can own at most 64 rows: N <= 64 * waves of the grid.
 inline bool gemv_applies(const void *row, const void *w, int N, int K)
 {
-    return K % 16 == 0 && K <= 14336 && N <= 64 * 4096 && aligned16(row) && aligned16(w) && !getenv("VTL_HIP_NO_GEMV");
+    return K % 16 == 0 && K <= 14336 && N <= 64 * gemv_max_waves(K) && aligned16(row) && aligned16(w) &&
+           !tuning().no_gemv;
 }
 
 template <bool F32OUT>
@@ -1668,7 +1637,7 @@ int launch_gemm(const GemmArgs &g_in, hipStream_t st)
         const size_t b_bytes = (size_t)g.N * Kp;
         int8_t *ws = static_cast<int8_t *>(vtlhip::library_workspace(a_bytes + b_bytes, 2));
         if (!ws)
-            return VTL_HIP_ERR_OUT_OF_MEMORY;
+            return vtlhip::workspace_status();
         const int64_t ta = (int64_t)g.M * (Kp / 4), tb = (int64_t)g.N * (Kp / 4);
         if ((ta + 255) / 256 > 0x7fffffff || (tb + 255) / 256 > 0x7fffffff)
             return VTL_HIP_ERR_UNSUPPORTED;
@@ -1684,28 +1653,25 @@ int launch_gemm(const GemmArgs &g_in, hipStream_t st)
         g.K = Kp;
     }
     // one row: matrix-vector product (very short rows go to the small-product kernel)
-    if (g.M == 1 && g.K >= 256 && gemv_applies(g.A, g.Bt, g.N, g.K) &&
-        !getenv("VTL_HIP_GEMM_CONFIG") && !getenv("VTL_HIP_GEMM_SMALL"))
+    const Tuning &tn = tuning();
+    const bool config_set = tn.gemm_config >= 0, small_set = tn.gemm_small >= 0;
+    if (g.M == 1 && g.K >= 256 && gemv_applies(g.A, g.Bt, g.N, g.K) && !config_set && !small_set)
         return launch_gemv<false, F32OUT>(g, st);
-    if (gemv_rows_applies(g.A, g.Bt, g.M, g.N, g.K) && gemv_rows_faster(g.M, g.N, g.K) &&
-        !getenv("VTL_HIP_GEMM_CONFIG") && !getenv("VTL_HIP_GEMM_SMALL"))
+    if (gemv_rows_applies(g.A, g.Bt, g.M, g.N, g.K) && gemv_rows_faster(g.M, g.N, g.K) && !config_set && !small_set)
         return launch_gemv_rows<false, F32OUT>(g, st);
-    if (g.K % 256 == 0 && g.M <= 32 && g.N >= 2048 && !getenv("VTL_HIP_GEMM_CONFIG"))
+    if (g.K % 256 == 0 && g.M <= 32 && g.N >= 2048 && !config_set)
         return launch_skinny<F32OUT>(g, st);  // weight streaming: enough row blocks to fill the chip
     const int64_t t32 = (int64_t)((g.M + 31) / 32) * ((g.N + 31) / 32);
-    const char *small_env = getenv("VTL_HIP_GEMM_SMALL");   // "1" / "0" force the choice (tests, tuning)
-    if (small_env ? atoi(small_env) != 0 : (t32 <= 64 && g.K <= 2048)) {
+    // VTL_HIP_GEMM_SMALL 1 / 0 forces the choice (tests, tuning)
+    if (small_set ? tn.gemm_small != 0 : (t32 <= 64 && g.K <= 2048)) {
         hipLaunchKernelGGL((gemm_i8_small_kernel<F32OUT>), dim3((unsigned)t32), dim3(256), 0, st, g);
         return check_launch("gemm_i8_small_kernel");
     }
     int idx, splits;
     choose_config(g.M, g.N, g.K, idx, splits);
-    if (const char *force = getenv("VTL_HIP_GEMM_CONFIG")) {  // tuning knob: "<tile index>,<splits>"
-        int fi = -1, fs = 1;
-        if (sscanf(force, "%d,%d", &fi, &fs) >= 1 && fi >= 0 && fi < kNumTileConfigs) {
-            idx = fi;
-            splits = fs;
-        }
+    if (config_set && tn.gemm_config < kNumTileConfigs) {  // tuning knob VTL_HIP_GEMM_CONFIG "<tile index>,<splits>"
+        idx = tn.gemm_config;
+        splits = tn.gemm_splits;
     }
     return launch_config<F32OUT>(idx, g, splits, st);
 }
@@ -1722,14 +1688,6 @@ int check_gemm_args(const void *A, const void *Bt, const void *out, int M, int N
 }  // namespace
 
 extern "C" {
-
-int vtl_hip_probe_mfma_i8(const int8_t *operands, int iterations, int32_t *sink)
-{
-    if (!operands || !sink || iterations < 0 || !aligned16(operands))
-        return VTL_HIP_ERR_INVALID_ARG;
-    hipLaunchKernelGGL(mfma_i8_probe_kernel, dim3(1024), dim3(256), 0, current_stream(), operands, iterations, sink);
-    return check_launch("mfma_i8_probe_kernel");
-}
 
 int vtl_hip_gemm_i8_i32(const int8_t *A, const int8_t *Bt, int32_t *C, int M, int N, int K)
 {
@@ -1780,7 +1738,7 @@ int vtl_hip_linear_i8_requant(const int8_t *A, const float *sa, int sa_per_row, 
         // a caller who wants the f32 rows anyway provides the staging: past 256 MiB of int32 sums
         // the two-pass route through Y needs no scratch of the library's
         !(Y && (size_t)M * (size_t)N * sizeof(int32_t) > ((size_t)256 << 20)) &&
-        !getenv("VTL_HIP_NO_FUSED_REQUANT")) {
+        !tuning().no_fused_requant) {
         // tile kernel leaves int32 sums, one row kernel does epilogue + quantization
         g.requant_codes = Yq;
         g.requant_scales = sy;
@@ -1793,7 +1751,7 @@ int vtl_hip_linear_i8_requant(const int8_t *A, const float *sa, int sa_per_row, 
     if (!Y) {
         Y = static_cast<float *>(vtlhip::library_workspace((size_t)M * (size_t)N * sizeof(float), 1));
         if (!Y)
-            return VTL_HIP_ERR_OUT_OF_MEMORY;
+            return vtlhip::workspace_status();
         g.out = Y;
     }
     st = launch_gemm<true>(g, current_stream());
@@ -1827,15 +1785,14 @@ int vtl_hip_linear_f32_dynquant(const float *X, const int8_t *Wq, const float *s
     if (workspace && (workspace_bytes < vtl_hip_linear_f32_dynquant_workspace(M, K) ||
                       (reinterpret_cast<uintptr_t>(workspace) & 15)))
         return VTL_HIP_ERR_INVALID_ARG;
-    if (M == 1 && gemv_applies(X, Wq, N, K) && !getenv("VTL_HIP_NO_FUSED_DECODE")) {
+    if (M == 1 && gemv_applies(X, Wq, N, K) && !tuning().no_fused_decode) {
         // a single token: quantized inside the matrix-vector kernel, one launch instead of two
         // (N = 14336, K = 4096: 9.5 us against 12.8 us).  The workspace stays unused.
         // VTL_HIP_NO_FUSED_DECODE forces the two-launch path (tests).
         GemmArgs g{nullptr, Wq, Y, nullptr, sw, bias, M, N, K, 1, 1, relu ? 1 : 0, 1, nullptr, X, 0};
         return launch_gemv<true, true>(g, current_stream());
     }
-    if (gemv_rows_applies(X, Wq, M, N, K) && gemv_rows_fused_quant_faster(M, N, K) &&
-        !getenv("VTL_HIP_NO_FUSED_DECODE")) {
+    if (gemv_rows_applies(X, Wq, M, N, K) && gemv_rows_fused_quant_faster(M, N, K) && !tuning().no_fused_decode) {
         // a few tokens and short rows: same, each workgroup quantizes the rows itself
         GemmArgs g{nullptr, Wq, Y, nullptr, sw, bias, M, N, K, 1, 1, relu ? 1 : 0, 1, nullptr, X, 0};
         return launch_gemv_rows<true, true>(g, current_stream());
@@ -1843,7 +1800,7 @@ int vtl_hip_linear_f32_dynquant(const float *X, const int8_t *Wq, const float *s
     if (!workspace) {   // no caller scratch: stage in the library's own buffer
         workspace = vtlhip::library_workspace(vtl_hip_linear_f32_dynquant_workspace(M, K), 1);
         if (!workspace)
-            return VTL_HIP_ERR_OUT_OF_MEMORY;
+            return vtlhip::workspace_status();
     }
     int8_t *xq = reinterpret_cast<int8_t *>(workspace);
     const size_t codes = (((size_t)M * (size_t)K) + 255) & ~(size_t)255;

@@ -442,7 +442,7 @@ int launch_split(MatmulArgs g, bool ta, bool tb, int splits, hipStream_t st)
     g.partial = static_cast<double *>(
         vtlhip::library_workspace((size_t)splits * (size_t)g.M * (size_t)g.N * sizeof(double)));
     if (!g.partial)
-        return VTL_HIP_ERR_OUT_OF_MEMORY;
+        return vtlhip::workspace_status();
     const bool whole = g.M % BM == 0 && g.N % BN == 0 && g.K % per == 0 && g.vec_a && g.vec_b;
     int rc = whole ? launch_tile_guard<T, TM, TN, WR, WC, false, true>(g, ta, tb, splits, st)
                    : launch_tile_guard<T, TM, TN, WR, WC, true, true>(g, ta, tb, splits, st);
@@ -491,10 +491,10 @@ int matmul_impl(const T *a, const T *b, T *c, const T *bias, int m, int n, int k
     const double t128 = (double)(c128 / 2) * (2.0 / 0.84) + (double)(c128 % 2) * (1.0 / 0.75);
     const double t64 = (double)c64 * 0.25 / (0.78 - 0.24 / (double)c64);
     // eight waves of 32x64 per 128x128 tile measured a few percent above four waves of 64x64
-    const char *tile_env = getenv("VTL_HIP_MATMUL_TILE");   // "128" / "64" force the tile (tuning, tests)
-    if (tile_env ? atoi(tile_env) == 128 : t128 <= t64)
+    const int tile_env = vtlhip::tuning().matmul_tile;   // VTL_HIP_MATMUL_TILE 128 / 64 forces the tile (tuning, tests)
+    if (tile_env ? tile_env == 128 : t128 <= t64)
         return launch_tile<T, 2, 4, 4, 2>(g, trans_a != 0, trans_b != 0, st);
-    const char *force = getenv("VTL_HIP_MATMUL_SPLITS");   // tuning and tests
+    const bool force = vtlhip::tuning().matmul_splits >= 0;   // VTL_HIP_MATMUL_SPLITS (tuning and tests)
     // Too few big tiles for the chip but a long K: cut K until about 512 big
     // workgroups exist (two per compute unit); measured 8-12 % faster than
     // the small tile with its own split (256x4096x11008: 428 -> 386 us).
@@ -505,7 +505,7 @@ int matmul_impl(const T *a, const T *b, T *c, const T *bias, int m, int n, int k
         if (sp > 1)
             return launch_split<T, 2, 4, 4, 2>(g, trans_a != 0, trans_b != 0, sp, st);
     }
-    int splits = force ? atoi(force) : 1;
+    int splits = force ? vtlhip::tuning().matmul_splits : 1;
     if (!force && small <= 512 && k >= 2048) {
         splits = (int)(1024 / small);
         if (splits > k / 512)
@@ -552,7 +552,7 @@ int colsum_impl(const T *x, int64_t rows, int64_t cols, T *out)
         partial = static_cast<double *>(
             vtlhip::library_workspace((size_t)splits * (size_t)cols * sizeof(double)));
         if (!partial)
-            return VTL_HIP_ERR_OUT_OF_MEMORY;
+            return vtlhip::workspace_status();
     }
     const dim3 grid((unsigned)col_blocks, (unsigned)splits);
     if (vec)

@@ -2,7 +2,10 @@
 // These are the calls the V-side HipStorage makes where CudaStorage calls
 // cudaMalloc / cudaMemcpy / cudaFree (storage/cuda_d_cuda.v:32-102).
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
+
+#include <atomic>
 
 #include "common.hpp"
 
@@ -33,23 +36,88 @@ int check_launch(const char *kernel_name)
     return VTL_HIP_OK;
 }
 
-void *library_workspace(size_t bytes, int slot)
+static Tuning g_tuning;
+static std::atomic<bool> g_tuning_read{false};
+
+static void read_tuning()
 {
-    constexpr int kMaxDevices = 64;
-    static void *bufs[3][kMaxDevices] = {};
-    static size_t caps[3][kMaxDevices] = {};
-    if (slot < 0 || slot > 2)
-        return nullptr;
-    void **buf = bufs[slot];
-    size_t *cap = caps[slot];
+    Tuning t;
+    auto flag = [](const char *name) { return getenv(name) != nullptr; };
+    auto number = [](const char *name, int unset) {
+        const char *v = getenv(name);
+        return v ? atoi(v) : unset;
+    };
+    t.no_gemv = flag("VTL_HIP_NO_GEMV");
+    t.gemv_rows = number("VTL_HIP_GEMV_ROWS", -1);
+    t.gemm_small = number("VTL_HIP_GEMM_SMALL", -1);
+    if (const char *v = getenv("VTL_HIP_GEMM_CONFIG")) {
+        int idx = -1, splits = 1;
+        // a value that does not parse still takes the launch off the special-case kernels
+        t.gemm_config = (sscanf(v, "%d,%d", &idx, &splits) >= 1 && idx >= 0) ? idx : 1 << 30;
+        t.gemm_splits = splits;
+    }
+    t.no_fused_requant = flag("VTL_HIP_NO_FUSED_REQUANT");
+    t.no_fused_decode = flag("VTL_HIP_NO_FUSED_DECODE");
+    t.matmul_tile = number("VTL_HIP_MATMUL_TILE", 0);
+    t.matmul_splits = number("VTL_HIP_MATMUL_SPLITS", -1);
+    g_tuning = t;
+    g_tuning_read.store(true, std::memory_order_release);
+}
+
+const Tuning &tuning()
+{
+    if (!g_tuning_read.load(std::memory_order_acquire))
+        read_tuning();
+    return g_tuning;
+}
+
+constexpr int kMaxDevices = 64;
+static thread_local int g_workspace_status = VTL_HIP_OK;
+
+static int current_device()
+{
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
         (void)hipGetLastError();
+        return -1;
+    }
+    return dev;
+}
+
+int workspace_status() { return g_workspace_status; }
+
+void *library_workspace(size_t bytes, int slot)
+{
+    static void *bufs[3][kMaxDevices] = {};
+    static size_t caps[3][kMaxDevices] = {};
+    g_workspace_status = VTL_HIP_OK;
+    if (slot < 0 || slot > 2) {
+        g_workspace_status = VTL_HIP_ERR_INVALID_ARG;
+        return nullptr;
+    }
+    void **buf = bufs[slot];
+    size_t *cap = caps[slot];
+    const int dev = current_device();
+    if (dev < 0) {
+        g_workspace_status = VTL_HIP_ERR_NO_DEVICE;
         return nullptr;
     }
     if (bytes > cap[dev]) {
+        // Growing frees the old buffer, which kernels of any stream may still use, and allocates:
+        // neither is possible while the current stream records a graph.
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(current_stream(), &capturing) != hipSuccess)
+            (void)hipGetLastError();
+        if (capturing != hipStreamCaptureStatusNone) {
+            snprintf(g_last_error, sizeof(g_last_error),
+                     "library scratch would have to grow to %zu bytes during a stream capture: run the call once "
+                     "before capturing",
+                     bytes);
+            g_workspace_status = VTL_HIP_ERR_UNSUPPORTED;
+            return nullptr;
+        }
         if (buf[dev]) {
-            (void)hipStreamSynchronize(current_stream());
+            (void)hipDeviceSynchronize();   // every stream: the buffer is shared by all of them
             (void)hipFree(buf[dev]);
             buf[dev] = nullptr;
             cap[dev] = 0;
@@ -58,6 +126,7 @@ void *library_workspace(size_t bytes, int slot)
         if (hipMalloc(&buf[dev], want) != hipSuccess) {
             (void)hipGetLastError();
             buf[dev] = nullptr;
+            g_workspace_status = VTL_HIP_ERR_OUT_OF_MEMORY;
             return nullptr;
         }
         cap[dev] = want;
@@ -243,6 +312,12 @@ const char *vtl_hip_strerror(int status)
 }
 
 const char *vtl_hip_last_error(void) { return g_last_error; }
+
+int vtl_hip_reload_env(void)
+{
+    read_tuning();
+    return VTL_HIP_OK;
+}
 
 const char *vtl_hip_version(void) { return "vtlhip 0.1 (gfx950)"; }
 

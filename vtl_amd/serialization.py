@@ -54,7 +54,7 @@ def linear_layer_entry(layer: QuantLinearLayer, in_shape, with_quantized: bool =
     """(LayerDef, SerializedLayer) dictionaries of one Linear layer."""
     out_f, in_f = layer.weights.shape
     layer_def = {"layer_type": "LinearLayer", "in_shape": [int(d) for d in in_shape],
-                 "config": {"out_features": int(out_f), "in_features": int(in_f)}}
+                 "config": {"in_features": int(in_f), "out_features": int(out_f)}}
     weights = {"weight": encode_tensor(layer.weights), "bias": encode_tensor(layer.bias)}
     if with_quantized:
         qw = layer.quantized()                      # device-resident codes and scales
@@ -65,9 +65,14 @@ def linear_layer_entry(layer: QuantLinearLayer, in_shape, with_quantized: bool =
 
 def save_model(path: str, layers, input_shape, with_quantized: bool = True, epoch: int = 0,
                loss: float = 0.0) -> None:
-    """Write a model file for a stack of QuantLinearLayer / "relu" entries."""
-    defs, data = [], []
-    shape = list(input_shape)
+    """Write a model file for a stack of QuantLinearLayer / "relu" entries behind
+    an input layer of `input_shape`, as Sequential.save_checkpoint does
+    (nn/models/serialization.v:108-124): the input layer is layer 0 with an empty
+    in_shape and its dimensions in the config (sequential_info.v:43-49), every
+    later layer records the output shape of the layer before it."""
+    shape = [int(d) for d in input_shape]
+    defs = [{"layer_type": "InputLayer", "in_shape": [], "config": {f"shape_{i}": d for i, d in enumerate(shape)}}]
+    data = [{"weights": {}}]
     for l in layers:
         if isinstance(l, QuantLinearLayer):
             d, w = linear_layer_entry(l, shape, with_quantized)
