@@ -161,6 +161,24 @@ int vtl_hip_linear_f32_dynquant(const float *X, const int8_t *Wq, const float *s
                                 const float *bias, float *Y, int M, int N, int K, int relu,
                                 void *workspace, size_t workspace_bytes);
 
+/* vtl_hip_linear_f32_dynquant for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc).  No counterpart in the reference.  Same arguments, arithmetic
+ * and bits as vtl_hip_linear_f32_dynquant with workspace == NULL, but every
+ * byte the call stages (activation codes and row scales, int32 partial sums
+ * of a K split, repacked operands) lives in a static 32 MiB array that is part
+ * of the library's code object, one per device: the call makes no hipMalloc /
+ * hipFree.  A shape whose staging does not fit returns VTL_HIP_ERR_UNSUPPORTED
+ * (vtl_hip_last_error() says how many bytes were missing) and leaves Y
+ * untouched.  All calls on a device share that device's array, which keeps
+ * the previous call's contents: calls that overlap on one device (several
+ * streams, several host threads) race; calls on one stream are ordered.
+ * vtl_hip_set_device resolves the array's device address, so a process that
+ * captures graphs should call it (or this entry point once) beforehand. */
+int vtl_hip_linear_f32_dynquant_noalloc(const float *X, const int8_t *Wq, const float *sw,
+                                        const float *bias, float *Y, int M, int N, int K,
+                                        int relu);
+
 /* ---- f32 / f64 matmul with f64 accumulation ------------------------------ */
 
 /* C[M,N] = op(A) . op(B) with every product and sum in f64 and one rounding

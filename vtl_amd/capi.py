@@ -49,6 +49,7 @@ SIGNATURES = {
     "vtl_hip_linear_i8_requant": (_ci, [_vp, _vp, _ci, _vp, _vp, _ci, _vp, _ci, _vp, _vp, _vp, _ci, _ci, _ci]),
     "vtl_hip_linear_f32_dynquant_workspace": (_sz, [_ci, _ci]),
     "vtl_hip_linear_f32_dynquant": (_ci, [_vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp, _sz]),
+    "vtl_hip_linear_f32_dynquant_noalloc": (_ci, [_vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci]),
     "vtl_hip_matmul_f32": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci]),
     "vtl_hip_matmul_f64": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _ci]),
     "vtl_hip_linear_f32": (_ci, [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci]),

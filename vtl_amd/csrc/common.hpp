@@ -30,9 +30,23 @@ bool launch_copy(void *dst, const void *src, size_t bytes, hipStream_t st);
 // when the allocation fails.
 void *library_workspace(size_t bytes, int slot = 0);
 // Why the last library_workspace() call of this thread returned nullptr
-// (VTL_HIP_ERR_OUT_OF_MEMORY, or VTL_HIP_ERR_UNSUPPORTED when the buffer would
-// have to grow during a stream capture).
+// (VTL_HIP_ERR_OUT_OF_MEMORY, or VTL_HIP_ERR_UNSUPPORTED when the request does
+// not fit the static scratch or would have to allocate during a stream capture).
 int workspace_status();
+
+// Static per-device scratch for the entry point that allocates nothing, and the
+// scope during which library_workspace() serves from it.  static_scratch()
+// returns the device address of the current device's array (nullptr on error).
+constexpr size_t kStaticScratchBytes = size_t(32) << 20;
+void *static_scratch();
+struct ScratchArena {
+    char *base;
+    size_t capacity, used = 0;
+    ScratchArena(void *base_, size_t capacity_);
+    ~ScratchArena();
+    ScratchArena(const ScratchArena &) = delete;
+    ScratchArena &operator=(const ScratchArena &) = delete;
+};
 
 // Tuning and test switches, taken from the environment once (first use) and
 // again only when vtl_hip_reload_env() is called: the dispatch path of a launch

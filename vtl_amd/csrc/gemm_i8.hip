@@ -1812,4 +1812,18 @@ int vtl_hip_linear_f32_dynquant(const float *X, const int8_t *Wq, const float *s
     return launch_gemm<true>(g, current_stream());
 }
 
+int vtl_hip_linear_f32_dynquant_noalloc(const float *X, const int8_t *Wq, const float *sw, const float *bias,
+                                        float *Y, int M, int N, int K, int relu)
+{
+    void *base = vtlhip::static_scratch();   // device address of this device's array, resolved once
+    if (!base)
+        return VTL_HIP_ERR_RUNTIME;
+    // Everything the call stages - activation codes and row scales, partial sums of a K split,
+    // repacked operands - is cut from the static array in the order it is asked for; a call that
+    // needs more than the array holds returns VTL_HIP_ERR_UNSUPPORTED (kernels that only fill
+    // earlier pieces of the scratch may have been enqueued by then; Y is not written).
+    vtlhip::ScratchArena arena(base, vtlhip::kStaticScratchBytes);
+    return vtl_hip_linear_f32_dynquant(X, Wq, sw, bias, Y, M, N, K, relu, nullptr, 0);
+}
+
 }  // extern "C"

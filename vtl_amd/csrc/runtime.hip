@@ -71,8 +71,16 @@ const Tuning &tuning()
     return g_tuning;
 }
 
+// ---- scratch for callers that cannot allocate --------------------------------
+// One array per device, part of the code object, so it exists from the moment
+// the library is loaded on a device until the process ends.  Host code never
+// uses the array's name as an address: static_scratch() asks the runtime for
+// the device address (once per device) and everything else goes through that
+// pointer.
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 constexpr int kMaxDevices = 64;
-static thread_local int g_workspace_status = VTL_HIP_OK;
+static void *g_scratch_ptr[kMaxDevices] = {};
 
 static int current_device()
 {
@@ -84,6 +92,35 @@ static int current_device()
     return dev;
 }
 
+void *static_scratch()
+{
+    const int dev = current_device();
+    if (dev < 0)
+        return nullptr;
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) {
+            (void)record_hip_error(e, "hipGetSymbolAddress(scratch)");
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = ptr;
+    }
+    return g_scratch_ptr[dev];
+}
+
+// While a ScratchArena is alive on this thread, library_workspace() hands out
+// consecutive pieces of it instead of the library's own growing buffers.
+static thread_local ScratchArena *g_arena = nullptr;
+static thread_local int g_workspace_status = VTL_HIP_OK;
+
+ScratchArena::ScratchArena(void *base_, size_t capacity_) : base(static_cast<char *>(base_)), capacity(capacity_)
+{
+    g_arena = this;
+}
+
+ScratchArena::~ScratchArena() { g_arena = nullptr; }
+
 int workspace_status() { return g_workspace_status; }
 
 void *library_workspace(size_t bytes, int slot)
@@ -94,6 +131,19 @@ void *library_workspace(size_t bytes, int slot)
     if (slot < 0 || slot > 2) {
         g_workspace_status = VTL_HIP_ERR_INVALID_ARG;
         return nullptr;
+    }
+    if (g_arena) {
+        const size_t take = (bytes + 255) & ~(size_t)255;
+        if (take > g_arena->capacity - g_arena->used) {
+            snprintf(g_last_error, sizeof(g_last_error),
+                     "call needs %zu more bytes of scratch, the static scratch of %zu bytes has %zu left", take,
+                     g_arena->capacity, g_arena->capacity - g_arena->used);
+            g_workspace_status = VTL_HIP_ERR_UNSUPPORTED;
+            return nullptr;
+        }
+        void *p = g_arena->base + g_arena->used;
+        g_arena->used += take;
+        return p;
     }
     void **buf = bufs[slot];
     size_t *cap = caps[slot];
@@ -162,6 +212,7 @@ int vtl_hip_set_device(int device_id)
     if (device_id < 0 || device_id >= c)
         return VTL_HIP_ERR_NO_DEVICE;
     VTL_HIP_TRY(hipSetDevice(device_id));
+    (void)static_scratch();   // resolved here so that a later call under stream capture finds it ready
     return VTL_HIP_OK;
 }
 
