@@ -272,7 +272,7 @@ def test_forced_split_k_is_exact(hip, knobs, k):
     ref = oracle.gemm_i8_i32(a, bt, threads=CPU_THREADS)
     want = oracle.epilogue(ref, sa, sb, bias)
     A, B, dsa, dsb, dbias = dev(a), dev(bt), dev(sa), dev(sb), dev(bias)
-    for idx in range(6):
+    for idx in range(8):
         for splits in (1, 2, 3, 8):
             knobs.setenv("VTL_HIP_GEMM_CONFIG", f"{idx},{splits}")
             assert np.array_equal(_gemm(a, bt), ref), (idx, splits)
