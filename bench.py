@@ -32,10 +32,32 @@ PEAK_INT8_TOPS = 5000.0      # dense int8 MFMA, MI355X published
 PEAK_HBM_GBPS = 8000.0       # HBM3E, MI355X published
 PEAK_FP64_TFLOPS = 78.6      # dense f64 MFMA, MI355X published
 
-# HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# script, each counter scaled by its reading for the 1 GiB copy_kernel (x2.000 and
-# x0.999); the summary of those runs is kept with the other profiler summaries.
-PMC_TRAFFIC_BYTES = {"linear": 168.1e6, "quantize": 1342.6e6, "dequantize": 1342.7e6, "linear_f32": 866.2e6}
+TRAFFIC_RECORDS = os.path.join(ROOT, "profiles", "bench_pmc_traffic.md")
+
+
+def measured_traffic(name: str):
+    """HBM-side bytes per launch of the kernel behind `name`, from the committed summary of
+    the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script (each counter scaled by
+    its reading for the 1 GiB copy kernel).  A record names the kernel's source file and the
+    SHA-256 of that file when the counters were read; if the file has changed since, the
+    figure is stale and None is reported instead."""
+    import hashlib
+    try:
+        lines = open(TRAFFIC_RECORDS).read().splitlines()
+    except OSError:
+        return None
+    for line in lines:
+        if not line.startswith("record:"):
+            continue
+        rec = dict(kv.split("=", 1) for kv in line[len("record:"):].split())
+        if rec.get("name") != name:
+            continue
+        try:
+            digest = hashlib.sha256(open(os.path.join(ROOT, rec["source"]), "rb").read()).hexdigest()
+        except OSError:
+            return None
+        return float(rec["bytes"]) if digest.startswith(rec["sha256"]) else None
+    return None
 
 
 class Timer:
@@ -108,10 +130,11 @@ def bench_linear(timer: Timer, steps: int, warmup: int, cpu: bool):
                      "achieved": ops / (kernel_ms * 1e-3) / 1e12, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                      "frac": ops / (kernel_ms * 1e-3) / 1e12 / PEAK_INT8_TOPS,
                      "kernel_us": kernel_ms * 1e3, "algorithmic_ops": ops,
-                     "traffic": PMC_TRAFFIC_BYTES["linear"]},
+                     "traffic": measured_traffic("linear")},
     }
     if cpu:
         import oracle  # CPU baseline leg only
+        flags = oracle.use_native_build()
         rows = m       # the whole workload once: a few seconds on one host core
         t0 = time.perf_counter()
         ref = oracle.linear_i8_f32(a[:rows], sa[:rows], bt, sb, bias, threads=1)
@@ -124,7 +147,7 @@ def bench_linear(timer: Timer, steps: int, warmup: int, cpu: bool):
         got = Y.cpu()[:rows]
         res["parity_sample_bit_exact"] = bool(np.array_equal(got, ref))
         res["cpu_baseline"] = {"value": 2.0 * rows * n * k / dt1 / 1e12, "unit": "TOPS", "cores": 1,
-                               "kind": "port",
+                               "kind": "port", "build": flags,
                                "sample": f"{rows} of {m} rows of A against all of Bt, {dt1:.1f} s, 1 thread"}
         res["cpu_baseline_all_cores"] = {"value": 2.0 * rows_mt * n * k / dtn / 1e12, "unit": "TOPS",
                                          "cores": threads, "kind": "port",
@@ -164,10 +187,11 @@ def bench_quant(timer: Timer, steps: int, warmup: int, cpu: bool):
             "config": {"workload": f"configs[1]: per-row {name} of f32 [16384,16384], seed 1"},
             "roofline": {"kernel": kern, "bound": "hbm", "achieved": gbps, "peak": PEAK_HBM_GBPS,
                          "unit": "GB/s", "frac": gbps / PEAK_HBM_GBPS, "kernel_us": kernel_ms * 1e3,
-                         "algorithmic_bytes": algo_bytes, "traffic": PMC_TRAFFIC_BYTES[name]},
+                         "algorithmic_bytes": algo_bytes, "traffic": measured_traffic(name)},
         }
     if cpu:
         import oracle  # CPU baseline leg only
+        oracle.use_native_build()
         sample = rows   # the whole tensor once: under a second per pass on one host core
         threads = oracle.max_threads()
         t0 = time.perf_counter()
@@ -180,6 +204,9 @@ def bench_quant(timer: Timer, steps: int, warmup: int, cpu: bool):
         t0 = time.perf_counter()
         oracle.quantize(x[:big], True, threads=threads)
         dqn = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        oracle.dequantize(qr, sr, True, threads=threads)
+        ddn = time.perf_counter() - t0
         sample_bytes = sample * cols * 5.0 + sample * 4.0
         out["quantize"]["cpu_baseline"] = {"value": sample_bytes / dq1 / 1e9, "unit": "GB/s", "cores": 1,
                                            "kind": "port", "sample": f"first {sample} rows, {dq1:.2f} s"}
@@ -188,6 +215,9 @@ def bench_quant(timer: Timer, steps: int, warmup: int, cpu: bool):
             "kind": "port", "sample": f"first {big} rows, {dqn:.2f} s, OpenMP"}
         out["dequantize"]["cpu_baseline"] = {"value": sample_bytes / dd1 / 1e9, "unit": "GB/s", "cores": 1,
                                              "kind": "port", "sample": f"first {sample} rows, {dd1:.2f} s"}
+        out["dequantize"]["cpu_baseline_all_cores"] = {
+            "value": sample_bytes / ddn / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"first {sample} rows, {ddn:.2f} s, OpenMP"}
         out["quantize"]["parity_sample_bit_exact"] = bool(
             np.array_equal(Q.cpu()[:sample], qr) and np.array_equal(S.cpu()[:sample], sr))
         out["dequantize"]["parity_sample_bit_exact"] = bool(np.array_equal(D.cpu()[:sample], dr))
@@ -196,7 +226,7 @@ def bench_quant(timer: Timer, steps: int, warmup: int, cpu: bool):
     return out
 
 
-def bench_other_configs(timer: Timer, steps: int, warmup: int):
+def bench_other_configs(timer: Timer, steps: int, warmup: int, cpu: bool = False):
     """Timings of the remaining configurations (parity for them is in tests/):
     configs[0] MNIST-MLP first layer, configs[3] decode-shaped linear with
     per-token quantization on the fly, configs[4] 3-layer int8 MLP chain."""
@@ -219,7 +249,32 @@ def bench_other_configs(timer: Timer, steps: int, warmup: int):
     def c1():
         capi.call("vtl_hip_quantize_f32_i8", X.ptr, 64, 784, 0, Xq.ptr, Sx.ptr)
         capi.call("vtl_hip_linear_i8_f32", Xq.ptr, Sx.ptr, 0, Wq.ptr, Sw.ptr, 0, B.ptr, Y.ptr, 64, 256, 784, 0)
-    out["configs[0] mnist first layer [64,784]x[256,784]^T"] = {"us": timed(c1), "ops": 2.0 * 64 * 784 * 256}
+    c0 = {"us": timed(c1), "ops": 2.0 * 64 * 784 * 256}
+    if cpu:
+        # The reference's own CPU-runnable case, timed on the host beside it: (i) the reference's
+        # existing f32 Linear restated (operands widened to f64, f64 product, one rounding to
+        # f32, bias added in f32: la/la.v:44-53, nn/layers/linear_forward_f32.v:16-18) and (ii) the
+        # int8 path of this build on the CPU oracle (per-tensor quantize of x, int8 linear).
+        import oracle  # CPU baseline leg only
+        oracle.use_native_build()
+        wq_h, sw_h = oracle.quantize(w, False)
+
+        def best_of(fn, reps=20):
+            ts = []
+            for _ in range(reps):
+                t0 = time.perf_counter()
+                fn()
+                ts.append(time.perf_counter() - t0)
+            return float(np.median(ts)) * 1e6
+
+        def int8_cpu():
+            xq_h, sx_h = oracle.quantize(x, False)
+            return oracle.linear_i8_f32(xq_h, sx_h, wq_h, sw_h, b.reshape(-1), threads=1)
+        c0["cpu_f32_linear_via_f64_us"] = best_of(lambda: oracle.linear_f32_via_f64(x, w, b.reshape(-1)))
+        c0["cpu_int8_path_us"] = best_of(int8_cpu)
+        c0["cpu_note"] = "one host thread, median of 20; " + oracle.build_flags()
+        c0["parity_bit_exact"] = bool(np.array_equal(Y.cpu(), int8_cpu()))
+    out["configs[0] mnist first layer [64,784]x[256,784]^T"] = c0
     for h in (X, W, B, Wq, Sw, Xq, Sx, Y):
         h.release()
 
@@ -253,10 +308,14 @@ def bench_other_configs(timer: Timer, steps: int, warmup: int):
             capi.call("vtl_hip_linear_f32_dynquant", X.ptr, w.ptr, Sw.ptr, None, Y.ptr, m, n, k, 0, ws.ptr, ws.size)
         us_hbm = timed(c4_streaming)
         algo = n * k + 16384.0 * m + 57344.0 * m + 57344.0     # Wq + X f32 + Y f32 + sw
-        dec[f"M={m}"] = {"us": us, "GB/s": algo / us / 1e3, "frac_of_hbm_peak": algo / us / 1e3 / PEAK_HBM_GBPS,
-                         "TOPS": 2.0 * m * n * k / us / 1e6, "algorithmic_bytes": algo,
-                         "weights_from_hbm": {"us": us_hbm, "GB/s": algo / us_hbm / 1e3,
-                                              "frac_of_hbm_peak": algo / us_hbm / 1e3 / PEAK_HBM_GBPS}}
+        # the roofline fraction is the one with the weights streaming from HBM; the figure with
+        # the 58.7 MB of weights resident in the last-level cache is kept beside it as a footnote
+        dec[f"M={m}"] = {"us": us_hbm, "GB/s": algo / us_hbm / 1e3,
+                         "roofline": {"bound": "hbm", "achieved": algo / us_hbm / 1e3, "peak": PEAK_HBM_GBPS,
+                                      "unit": "GB/s", "frac": algo / us_hbm / 1e3 / PEAK_HBM_GBPS},
+                         "TOPS": 2.0 * m * n * k / us_hbm / 1e6, "algorithmic_bytes": algo,
+                         "weights_in_last_level_cache": {"us": us, "GB/s": algo / us / 1e3,
+                                                         "note": "same weights every launch: not an HBM figure"}}
         capi.call("vtl_hip_sync")
         for h in (X, Y):
             h.release()
@@ -339,7 +398,7 @@ def bench_full_precision(timer: Timer, steps: int, warmup: int):
     out["linear_f32 (f64 accumulate) M=N=K=4096"] = {
         "us": us, "TFLOP/s": tf,
         "roofline": {"bound": "mfma", "achieved": tf, "peak": PEAK_FP64_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tf / PEAK_FP64_TFLOPS, "traffic": PMC_TRAFFIC_BYTES["linear_f32"],
+                     "frac": tf / PEAK_FP64_TFLOPS, "traffic": measured_traffic("linear_f32"),
                      "kernel": "matmul_f64acc_kernel<float, 2, 4, 4, 2, false, true, false, false>"}}
     for h in (X, W, B, Y):
         h.release()
@@ -444,7 +503,7 @@ def main() -> int:
         print(json.dumps({"full_precision": bench_full_precision(timer, args.steps, args.warmup)}))
         return 0
     if args.only == "other":
-        print(json.dumps({"other_configs": bench_other_configs(timer, args.steps, args.warmup)}))
+        print(json.dumps({"other_configs": bench_other_configs(timer, args.steps, args.warmup, cpu)}))
         return 0
     if args.only == "mfma":
         print(json.dumps({"mfma_only": bench_mfma_only(timer)}))
@@ -485,7 +544,7 @@ def main() -> int:
         line["roofline"]["frac_of_mfma_only_rate_on_these_operands"] = (
             line["roofline"]["achieved"] / line["mfma_only"]["uniform_random_operands"]["TOP/s"])
     if args.only == "all":
-        line["other_configs"] = bench_other_configs(timer, args.steps, args.warmup)
+        line["other_configs"] = bench_other_configs(timer, args.steps, args.warmup, cpu)
         line["full_precision"] = bench_full_precision(timer, args.steps, args.warmup)
     print(json.dumps(line))
     return 0

@@ -26,13 +26,41 @@ def build(force: bool = False) -> str:
     return _LIB_PATH
 
 
-def lib() -> C.CDLL:
+_NATIVE_PATH = os.path.join(_HERE, "_native", "libvtloracle_native.so")
+_flags = "-O3 -march=x86-64-v3 -ffp-contract=off -fopenmp (oracle/Makefile)"
+
+
+def use_native_build() -> str:
+    """For the CPU-baseline leg of bench.py: compile the same source for the CPU
+    of THIS machine (gcc -O3 -march=native -ffp-contract=off -fopenmp, about a
+    second) and make later calls use it.  The shipped library is built for a
+    generic x86-64-v3 target because it travels between machines.  Returns the
+    flags in use; keeps the shipped build when gcc is missing or fails."""
+    global _lib, _flags
+    os.makedirs(os.path.dirname(_NATIVE_PATH), exist_ok=True)
+    cmd = ["gcc", "-O3", "-march=native", "-ffp-contract=off", "-fno-fast-math", "-fopenmp", "-fPIC", "-std=c11",
+           "-shared", "-o", _NATIVE_PATH, os.path.join(_HERE, "vtl_oracle.c"), "-lm"]
+    try:
+        subprocess.run(cmd, check=True, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, timeout=120)
+    except (OSError, subprocess.SubprocessError):
+        return _flags
+    _lib = None
+    lib(_NATIVE_PATH)
+    _flags = "-O3 -march=native -ffp-contract=off -fopenmp (built on this host)"
+    return _flags
+
+
+def build_flags() -> str:
+    return _flags
+
+
+def lib(path: str | None = None) -> C.CDLL:
     global _lib
     if _lib is not None:
         return _lib
-    if not os.path.exists(_LIB_PATH):
+    if path is None and not os.path.exists(_LIB_PATH):
         build()
-    L = C.CDLL(_LIB_PATH)
+    L = C.CDLL(path or _LIB_PATH)
     i64, ci, vp, f32 = C.c_int64, C.c_int, C.c_void_p, C.c_float
     sig = {
         "vtl_ref_absmax_f32": (None, [vp, i64, i64, ci, vp]),

@@ -120,6 +120,55 @@ int main(int argc, char **argv)
         } catch (const std::invalid_argument &) {
         }
     }
+    // the session: weights quantized once and kept on the device, staging buffer reused,
+    // activations handed from layer to layer (autograd_hip/hip_session_d_hip.v)
+    {
+        const int H = 64, O = 24;
+        std::vector<float> w2((size_t)O * N), b2(O), w1b = w;
+        for (auto &v : w2) v = nd(rng) * 0.05f;
+        for (auto &v : b2) v = nd(rng) * 0.1f;
+        (void)H;
+        vtl::HipSession s;
+        s.init_device();
+        CHECK(s.enabled);
+        auto ref_linear = [&](const std::vector<float> &xin, int m, int k, const std::vector<float> &wf, int n,
+                              const std::vector<float> &bf, bool relu) {
+            std::vector<int8_t> wq(wf.size());
+            std::vector<float> sw(n), out((size_t)m * n);
+            vtl_ref_quantize_f32_i8(wf.data(), n, k, 1, wq.data(), sw.data());
+            vtl_ref_linear_f32_dynquant(xin.data(), wq.data(), sw.data(), bf.data(), out.data(), m, n, k, relu, 1);
+            return out;
+        };
+        auto y1 = s.linear_forward_f32(x, M, K, w, N, b, &w, nullptr);
+        void *ws_first = s.workspace.ptr;
+        void *codes_first = s.layers[0].w_q.data.ptr;
+        auto y1b = s.linear_forward_f32(x, M, K, w, N, b, &w, nullptr);
+        CHECK(s.layers.size() == 1 && s.quantize_count == 1);          // quantized once
+        CHECK(s.workspace.ptr == ws_first && s.layers[0].w_q.data.ptr == codes_first);
+        CHECK(y1 == y1b && y1 == ref_linear(x, M, K, w, N, b, false));
+        // an optimizer step replaces the weight tensor: same slot, new codes
+        for (auto &v : w1b) v = -v;
+        auto y1c = s.linear_forward_f32(x, M, K, w1b, N, b, &w, nullptr);
+        CHECK(s.layers.size() == 1 && s.quantize_count == 2);
+        CHECK(y1c == ref_linear(x, M, K, w1b, N, b, false));
+        // Linear -> ReLU -> Linear with the activation staying on the device
+        auto h = s.linear_forward_f32(x, M, K, w, N, b, &w, nullptr);
+        CHECK(s.has_pending);
+        auto h_dev = s.take_pending();
+        auto r = s.relu_forward_f32(std::move(h_dev));
+        std::vector<float> r_ref = h;
+        vtl_ref_relu_f32(r_ref.data(), (int64_t)r_ref.size());
+        CHECK(r == r_ref);
+        auto r_dev = s.take_pending();
+        auto out = s.linear_forward_f32(r, M, N, w2, O, b2, &w2, &r_dev);
+        CHECK(out == ref_linear(r_ref, M, N, w2, O, b2, false));
+        CHECK(s.layers.size() == 2);
+        // the whole chain with int8 hand-off equals the layer-by-layer result bit for bit
+        auto chain = s.mlp_forward_i8(x, M, {&w, &w2}, {&b, &b2}, {K, N, O}, {true, false});
+        auto h_relu = ref_linear(x, M, K, w, N, b, true);
+        CHECK(chain == ref_linear(h_relu, M, N, w2, O, b2, false));
+        s.release();
+    }
     // la.matmul and LinearGate.backward with f64 accumulation vs oracle: integer-valued
     // operands, for which every summation order gives the same bits
     {

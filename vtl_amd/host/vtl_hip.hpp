@@ -224,13 +224,49 @@ inline std::vector<float> linear_forward_hip_f32(const std::vector<float> &x, in
     HipStorage<float> b_dev;
     if (bias)
         b_dev = HipStorage<float>::from_cpu(*bias);
-    HipStorage<uint8_t> ws(vtl_hip_linear_f32_dynquant_workspace(m, k));
     HipTensor<float> y({m, n});
+    // null workspace: the library stages the activation codes in its own buffer
     hip_check(vtl_hip_linear_f32_dynquant((const float *)x_dev.data.ptr, (const int8_t *)wq.first.data.ptr,
                                           (const float *)wq.second.data.ptr, (const float *)b_dev.ptr,
-                                          (float *)y.data.ptr, m, n, k, relu ? 1 : 0, ws.ptr, ws.size),
+                                          (float *)y.data.ptr, m, n, k, relu ? 1 : 0, nullptr, 0),
               "vtl_hip_linear_f32_dynquant");
     return y.cpu();
+}
+
+// `linear_i8_hip(x_q, sx, w_q, sw, bias, relu) !&HipTensor[f32]`
+inline HipTensor<float> linear_i8_hip(const HipTensor<int8_t> &x_q, const HipTensor<float> &sx,
+                                      const HipTensor<int8_t> &w_q, const HipTensor<float> &sw,
+                                      const HipStorage<float> *bias, bool relu)
+{
+    int m, n, k;
+    matmul_shapes(x_q.shape, w_q.shape, m, n, k);
+    HipTensor<float> y({m, n}, HipParams{x_q.data.device_id});
+    hip_check(vtl_hip_linear_i8_f32((const int8_t *)x_q.data.ptr, (const float *)sx.data.ptr, sx.size == (size_t)m,
+                                    (const int8_t *)w_q.data.ptr, (const float *)sw.data.ptr, sw.size == (size_t)n,
+                                    bias ? (const float *)bias->ptr : nullptr, (float *)y.data.ptr, m, n, k,
+                                    relu ? 1 : 0),
+              "vtl_hip_linear_i8_f32");
+    return y;
+}
+
+// `linear_i8_requant_hip(x_q, sx, w_q, sw, bias, relu) !(&HipTensor[i8], &HipTensor[f32])`:
+// the hand-off between two int8 layers.
+inline std::pair<HipTensor<int8_t>, HipTensor<float>> linear_i8_requant_hip(
+    const HipTensor<int8_t> &x_q, const HipTensor<float> &sx, const HipTensor<int8_t> &w_q,
+    const HipTensor<float> &sw, const HipStorage<float> *bias, bool relu)
+{
+    int m, n, k;
+    matmul_shapes(x_q.shape, w_q.shape, m, n, k);
+    HipParams p{x_q.data.device_id};
+    HipTensor<int8_t> y_q({m, n}, p);
+    HipTensor<float> sy({m}, p);
+    hip_check(vtl_hip_linear_i8_requant((const int8_t *)x_q.data.ptr, (const float *)sx.data.ptr,
+                                        sx.size == (size_t)m, (const int8_t *)w_q.data.ptr,
+                                        (const float *)sw.data.ptr, sw.size == (size_t)n,
+                                        bias ? (const float *)bias->ptr : nullptr, relu ? 1 : 0,
+                                        (int8_t *)y_q.data.ptr, (float *)sy.data.ptr, nullptr, m, n, k),
+              "vtl_hip_linear_i8_requant");
+    return {std::move(y_q), std::move(sy)};
 }
 
 // `matmul_hip(a, b, trans_a, trans_b) !&HipTensor[T]`: la.matmul (la/la.v:38-55)
@@ -327,5 +363,147 @@ inline std::vector<std::vector<float>> linear_backward_hip_f32(const std::vector
               "vtl_hip_linear_backward_f32");
     return {dx.cpu(), dw.cpu(), bias_needs_grad ? db.to_array() : std::vector<float>((size_t)n, 0.0f)};
 }
+
+// `HipSession` (autograd_hip/hip_session_d_hip.v): per-Context device state of the
+// INT8 path - the staging buffer of the activation quantization, the int8 weights of
+// every layer that ran through it (quantized once; `slot` names the layer, `source`
+// the weight tensor the codes were made from, so a replaced tensor is re-quantized)
+// and the f32 rows the last layer left on the device for the next one.
+class HipSession {
+public:
+    struct QuantizedWeights {
+        const void *slot = nullptr, *source = nullptr, *bias_source = nullptr;
+        HipTensor<int8_t> w_q;
+        HipTensor<float> sw;
+        HipStorage<float> bias;
+    };
+    bool enabled = false;
+    bool keep_activations = true;   // VTL_HIP_ACTIVATIONS=1 in the V host
+    std::vector<QuantizedWeights> layers;
+    HipStorage<uint8_t> workspace;
+    HipTensor<float> pending;
+    bool has_pending = false;
+    int quantize_count = 0;         // how often weights were (re)quantized: for tests
+
+    void init_device()
+    {
+        int n = 0;
+        enabled = vtl_hip_device_count(&n) == VTL_HIP_OK && n > 0;
+    }
+    void release()
+    {
+        layers.clear();
+        workspace.release();
+        pending.release();
+        has_pending = false;
+    }
+    const HipStorage<uint8_t> &ensure_workspace(int m, int k)
+    {
+        const size_t need = vtl_hip_linear_f32_dynquant_workspace(m, k);
+        if (!workspace.ptr || workspace.size < need)
+            workspace = HipStorage<uint8_t>(need);
+        return workspace;
+    }
+    // `weights` / `bias` are the host tensors' storage; their addresses are the cache keys
+    QuantizedWeights &quantized(const void *slot, const std::vector<float> &weights, int n, int k,
+                                const std::vector<float> &bias)
+    {
+        QuantizedWeights *q = nullptr;
+        for (auto &l : layers)
+            if (l.slot == slot)
+                q = &l;
+        if (!q) {
+            layers.emplace_back();
+            q = &layers.back();
+            q->slot = slot;
+        }
+        if (q->source != (const void *)&weights || !q->w_q.data.ptr) {
+            auto w_dev = HipTensor<float>::from_host(weights, {n, k});
+            auto qs = quantize_i8(w_dev, 0);
+            q->w_q = std::move(qs.first);
+            q->sw = std::move(qs.second);
+            q->source = &weights;
+            quantize_count++;
+        }
+        if (q->bias_source != (const void *)&bias || !q->bias.ptr) {
+            q->bias = HipStorage<float>::from_cpu(bias);
+            q->bias_source = &bias;
+        }
+        return *q;
+    }
+    // `(mut s HipSession) linear_forward_f32(x, weights, bias, slot, input_gpu) !&vtl.Tensor[f32]`:
+    // host rows out; the device rows stay pending for the next layer.  `input_gpu` is a
+    // device activation taken from the previous layer (take_pending) or null.
+    std::vector<float> linear_forward_f32(const std::vector<float> &x, int m, int k,
+                                          const std::vector<float> &weights, int n,
+                                          const std::vector<float> &bias, const void *slot,
+                                          HipTensor<float> *input_gpu)
+    {
+        if (!enabled)
+            throw HipError("hip session disabled", VTL_HIP_ERR_NO_DEVICE);
+        if (x.size() != (size_t)m * k || weights.size() != (size_t)n * k)
+            throw std::invalid_argument("Invalid shapes for matrix multiplication");
+        pending.release();
+        has_pending = false;
+        QuantizedWeights &q = quantized(slot, weights, n, k, bias);
+        const HipStorage<uint8_t> &ws = ensure_workspace(m, k);
+        HipTensor<float> uploaded;
+        const HipTensor<float> *x_dev = input_gpu;
+        if (!x_dev) {
+            uploaded = HipTensor<float>::from_host(x, {m, k});
+            x_dev = &uploaded;
+        } else if (x_dev->shape != std::vector<int>{m, k}) {
+            throw std::invalid_argument("hip chain: input activation shape mismatch");
+        }
+        HipTensor<float> y({m, n});
+        hip_check(vtl_hip_linear_f32_dynquant((const float *)x_dev->data.ptr, (const int8_t *)q.w_q.data.ptr,
+                                              (const float *)q.sw.data.ptr, (const float *)q.bias.ptr,
+                                              (float *)y.data.ptr, m, n, k, 0, ws.ptr, ws.size),
+                  "vtl_hip_linear_f32_dynquant");
+        std::vector<float> host = y.cpu();
+        if (keep_activations) {
+            pending = std::move(y);
+            has_pending = true;
+        }
+        return host;
+    }
+    // `relu_forward_f32(x, input_gpu)`: ReLU in place on the device activation, kept pending
+    std::vector<float> relu_forward_f32(HipTensor<float> &&input_gpu)
+    {
+        relu_hip(input_gpu);
+        std::vector<float> host = input_gpu.cpu();
+        pending = std::move(input_gpu);
+        has_pending = true;
+        return host;
+    }
+    // `session_bind_hip_activation`: the pending activation moves to the caller (the Variable)
+    HipTensor<float> take_pending()
+    {
+        has_pending = false;
+        return std::move(pending);
+    }
+    // `mlp_forward_i8(x, weights, biases, relu_after, slots)`: the whole chain on the device,
+    // int8 codes handed from layer to layer, f32 rows of the last layer back to the host.
+    std::vector<float> mlp_forward_i8(const std::vector<float> &x, int m,
+                                      const std::vector<const std::vector<float> *> &weights,
+                                      const std::vector<const std::vector<float> *> &biases,
+                                      const std::vector<int> &dims, const std::vector<bool> &relu_after)
+    {
+        if (!enabled)
+            throw HipError("hip session disabled", VTL_HIP_ERR_NO_DEVICE);
+        const size_t nl = weights.size();
+        if (nl == 0 || biases.size() != nl || relu_after.size() != nl || dims.size() != nl + 1)
+            throw std::invalid_argument("mlp_forward_i8: one bias and ReLU flag per weight matrix expected");
+        auto x_dev = HipTensor<float>::from_host(x, {m, dims[0]});
+        auto cur = quantize_i8(x_dev, 0);
+        x_dev.release();
+        for (size_t i = 0; i + 1 < nl; i++) {
+            QuantizedWeights &q = quantized(weights[i], *weights[i], dims[i + 1], dims[i], *biases[i]);
+            cur = linear_i8_requant_hip(cur.first, cur.second, q.w_q, q.sw, &q.bias, relu_after[i]);
+        }
+        QuantizedWeights &q = quantized(weights[nl - 1], *weights[nl - 1], dims[nl], dims[nl - 1], *biases[nl - 1]);
+        return linear_i8_hip(cur.first, cur.second, q.w_q, q.sw, &q.bias, relu_after[nl - 1]).cpu();
+    }
+};
 
 }  // namespace vtl
