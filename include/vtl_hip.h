@@ -124,7 +124,9 @@ int vtl_hip_dequantize_i8_f32(const int8_t *q, const float *scale, int64_t rows,
  * gemm_cuda (tensor_cuda_d_cuda.v:155-177) with the second operand given
  * K-contiguous.  K <= 131072 so that |acc| <= K * 127^2 < 2^31.  Any K and any
  * alignment; K % 16 == 0 with A and Bt 16-byte aligned spares a repacking pass
- * through scratch memory that the library allocates. */
+ * through scratch memory that the library allocates.  Outputs of more than
+ * 2^32 elements are addressed in 64 bits; only min(M, 32) * N >= 2^32 (more
+ * than 2^27 columns) can return VTL_HIP_ERR_UNSUPPORTED. */
 int vtl_hip_gemm_i8_i32(const int8_t *A, const int8_t *Bt, int32_t *C, int M, int N, int K);
 
 /* Y[m,n] = fl(fl(f32(acc) * fl(sa[m] * sw[n])) + bias[n]), ReLU if relu != 0

@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import CPU_THREADS, dev
+from helpers import CPU_THREADS, d2h, dev, raw_device_buffer
 from vtl_amd import capi
 from vtl_amd.tensor import HipTensor, linear_i8_hip
 
@@ -138,3 +138,40 @@ def test_requantizing_linear_beyond_2_31_elements(hip, keep_f32):
             assert np.array_equal(gy, y_ref)
     for h in (A, W, SA, SW, B) + tuple(out):
         h.release()
+
+
+def test_wide_output_beyond_2_32_elements(hip, knobs):
+    """Maximum sizes: 260 x 16.9 M outputs (4.4e9 elements, 17.6 GB of f32).  Element offsets past
+    2^32 must be formed in 64 bits: whole rows from either side of every tile-row boundary are
+    compared with the oracle, and the one tile shape that cannot address such a row length
+    (256 rows x N >= 2^32) is refused rather than run."""
+    m, n, k = 260, (1 << 24) + 123000, 32
+    rng = np.random.default_rng(2024)
+    a = rng.integers(-127, 128, (m, k), dtype=np.int8)
+    bt = rng.integers(-127, 128, (n, k), dtype=np.int8)
+    sa = rng.uniform(0.01, 0.02, m).astype(np.float32)
+    sb = rng.uniform(0.01, 0.02, n).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    A, B, dsa, dsb, dbias = dev(a), dev(bt), dev(sa), dev(sb), dev(bias)
+    rows = [0, 31, 32, 127, 128, 255, 256, 259]
+    ref = oracle.gemm_i8_i32(a[rows], bt, threads=CPU_THREADS)
+    want = oracle.epilogue(ref, sa[rows], sb, bias, relu=True)
+
+    out = raw_device_buffer(m * n * 4)
+    capi.call("vtl_hip_gemm_i8_i32", A.ptr, B.ptr, out.ptr, m, n, k)
+    for i, r in enumerate(rows):
+        assert np.array_equal(d2h(out.ptr + r * n * 4, (n,), np.int32), ref[i]), r
+    capi.call("vtl_hip_linear_i8_f32", A.ptr, dsa.ptr, 1, B.ptr, dsb.ptr, 1, dbias.ptr, out.ptr, m, n, k, 1)
+    for i, r in enumerate(rows):
+        assert np.array_equal(d2h(out.ptr + r * n * 4, (n,), np.float32), want[i]), r
+
+    knobs.setenv("VTL_HIP_GEMM_CONFIG", "7,1")     # 256 x 256 tiles: 255 * N + 255 >= 2^32
+    assert capi.status("vtl_hip_gemm_i8_i32", A.ptr, B.ptr, out.ptr, m, n, k) == capi.ERR_UNSUPPORTED
+    knobs.setenv("VTL_HIP_GEMM_CONFIG", "5,1")     # 128 x 128 tiles still can
+    capi.call("vtl_hip_gemm_i8_i32", A.ptr, B.ptr, out.ptr, m, n, k)
+    for i, r in enumerate(rows):
+        assert np.array_equal(d2h(out.ptr + r * n * 4, (n,), np.int32), ref[i]), r
+    knobs.delenv("VTL_HIP_GEMM_CONFIG")
+    for h in (A, B, dsa, dsb, dbias):
+        h.release()
+    out.release()

@@ -1410,18 +1410,29 @@ struct TileConfig {
     int wgs_per_cu;     // workgroups that fit a compute unit's LDS together
 };
 constexpr TileConfig kTileConfigs[] = {
-    {32, 64, 357.f, 1}, {32, 128, 600.f, 2},
-    {64, 64, 388.f, 2},   // four stages
-    {64, 128, 608.f, 2},
-    {128, 64, 588.f, 1},  // four stages
+    {32, 64, 359.f, 1}, {32, 128, 480.f, 2},
+    {64, 64, 420.f, 2},   // four stages
+    {64, 128, 693.f, 2},
+    {128, 64, 560.f, 1},  // four stages
     {128, 128, 900.f, 2},
-    {128, 128, 800.f, 1},  // four stages: alone on its compute unit, for launches of one round
+    {128, 128, 760.f, 1},  // four stages: alone on its compute unit, for launches of one round
     {256, 256, 1800.f, 1}};
 constexpr int kNumTileConfigs = 8;
+
+// The epilogue addresses a tile's elements as a 32-bit offset (row in tile x N
+// + column in tile) from the tile's origin: a tile shape qualifies only while
+// the largest such offset fits.
+inline bool tile_offsets_fit(const TileConfig &c, int M, int N)
+{
+    const int64_t rows = c.bm < M ? c.bm : M;
+    return rows * (int64_t)N + c.bn <= (int64_t)0xffffffffLL;
+}
 
 template <bool F32OUT>
 int launch_config(int idx, const GemmArgs &g, int splits, hipStream_t st)
 {
+    if (idx < 0 || idx >= kNumTileConfigs || !tile_offsets_fit(kTileConfigs[idx], g.M, g.N))
+        return VTL_HIP_ERR_UNSUPPORTED;  // more than 2^32 / 32 output columns: no tile shape qualifies
     switch (idx) {
     case 0: return launch_dma<32, 64, 128, 8, 1, 2, F32OUT>(g, splits, st);
     case 1: return launch_dma<32, 128, 128, 4, 1, 4, F32OUT>(g, splits, st);
@@ -1439,20 +1450,27 @@ int launch_config(int idx, const GemmArgs &g, int splits, hipStream_t st)
 //   latency:    rounds of workgroups over the resident slots x K steps per workgroup x step cost
 //   throughput: all K steps of all workgroups x step cost / 256 compute units
 // plus, for split K, the extra launch and the pass over the partial sums.
-// The constants were fitted (random search, least mean log regret) to an
-// exhaustive timing sweep of every tile and split count over 64 shapes, the
-// shapes of the decode and MLP-chain workloads weighted six-fold (mean regret
-// 1.3 %, worst 14 % at 1000x3000x2048).
+// The constants were fitted (random search, least mean log regret) to two
+// exhaustive timing sweeps of every tile and split count over 72 shapes - one
+// with the same weights every launch (up to 256 MB of them then stay in the
+// last-level cache), one with the weights taken from enough copies in turn that
+// every launch streams them from HBM, since which tile wins can depend on that
+// (160x14336x4096: 64x128 tiles take 20.5 us cached and 30.5 us from HBM,
+// 128x128 tiles 22.6 and 25.4) - the shapes of the decode and MLP-chain
+// workloads weighted six-fold.  Mean regret 1.7 % cached and 0.6 % from HBM,
+// worst 19 % (192x8192x8192 cached).
 void choose_config(int M, int N, int K, int &best_idx, int &best_splits)
 {
     const int kt_all = (K + 127) / 128;
     float best = 3.0e38f;
-    best_idx = kNumTileConfigs - 1;
+    best_idx = -1;  // stays so when no tile shape can address the output (see tile_offsets_fit)
     best_splits = 1;
     for (int i = 0; i < kNumTileConfigs; i++) {
         const TileConfig &c = kTileConfigs[i];
         if (i > 0 && kTileConfigs[i - 1].bm >= M && c.bm > kTileConfigs[i - 1].bm)
             break;  // a taller tile would only add padding rows
+        if (!tile_offsets_fit(c, M, N))
+            continue;
         const int64_t tiles = (int64_t)((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
         // More than one round of 256x256 tiles with a short K: each round pays the long fill and
         // the 256 KiB store of a tile that owns its compute unit, while two 128x128 tiles per
@@ -1465,12 +1483,12 @@ void choose_config(int M, int N, int K, int &best_idx, int &best_splits)
                 break;
             const int64_t rounds = (tiles * s + 256 * c.wgs_per_cu - 1) / (256 * c.wgs_per_cu);
             const int steps = (kt_all + s - 1) / s;
-            const float fixed = c.bm == 256 ? 6000.f : 4000.f;   // fill and store of one workgroup
+            const float fixed = c.bm == 256 ? 8000.f : 6000.f;   // fill and store of one workgroup
             const float latency = (float)rounds * ((float)steps * c.step_cycles + fixed);
             const float throughput = (float)tiles * (float)s * (float)steps * c.step_cycles / 256.f + fixed;
             float cost = latency > throughput ? latency : throughput;
             if (s > 1)
-                cost += 4500.f + (float)s * (float)M * (float)N * 4.0f / 1500.f;
+                cost += 4500.f + (float)s * (float)M * (float)N * 4.0f / 1350.f;
             if (cost < best) {
                 best = cost;
                 best_idx = i;
