@@ -1410,13 +1410,13 @@ struct TileConfig {
     int wgs_per_cu;     // workgroups that fit a compute unit's LDS together
 };
 constexpr TileConfig kTileConfigs[] = {
-    {32, 64, 359.f, 1}, {32, 128, 480.f, 2},
-    {64, 64, 420.f, 2},   // four stages
-    {64, 128, 693.f, 2},
-    {128, 64, 560.f, 1},  // four stages
-    {128, 128, 900.f, 2},
-    {128, 128, 760.f, 1},  // four stages: alone on its compute unit, for launches of one round
-    {256, 256, 1800.f, 1}};
+    {32, 64, 441.f, 1}, {32, 128, 600.f, 2},
+    {64, 64, 432.f, 2},   // four stages
+    {64, 128, 611.f, 2},
+    {128, 64, 576.f, 1},  // four stages
+    {128, 128, 1050.f, 2},
+    {128, 128, 665.f, 1},  // four stages, eight waves: alone on its compute unit, for launches of one round
+    {256, 256, 2200.f, 1}};
 constexpr int kNumTileConfigs = 8;
 
 // The epilogue addresses a tile's elements as a 32-bit offset (row in tile x N
@@ -1440,7 +1440,7 @@ int launch_config(int idx, const GemmArgs &g, int splits, hipStream_t st)
     case 3: return launch_dma<64, 128, 128, 3, 2, 2, F32OUT>(g, splits, st);
     case 4: return launch_dma<128, 64, 128, 4, 2, 2, F32OUT>(g, splits, st);
     case 5: return launch_dma<128, 128, 128, 2, 2, 2, F32OUT>(g, splits, st);
-    case 6: return launch_dma<128, 128, 128, 4, 2, 2, F32OUT>(g, splits, st);
+    case 6: return launch_dma<128, 128, 128, 4, 2, 4, F32OUT>(g, splits, st);
     default: return launch_dma<256, 256, 128, 2, 2, 4, F32OUT>(g, splits, st);
     }
 }
@@ -1457,8 +1457,8 @@ int launch_config(int idx, const GemmArgs &g, int splits, hipStream_t st)
 // every launch streams them from HBM, since which tile wins can depend on that
 // (160x14336x4096: 64x128 tiles take 20.5 us cached and 30.5 us from HBM,
 // 128x128 tiles 22.6 and 25.4) - the shapes of the decode and MLP-chain
-// workloads weighted six-fold.  Mean regret 1.7 % cached and 0.6 % from HBM,
-// worst 19 % (192x8192x8192 cached).
+// workloads weighted six-fold.  Mean regret 1.2 % cached and 0.7 % from HBM,
+// worst 13 % (192x8192x8192 and 6144x6144x2048 cached).
 void choose_config(int M, int N, int K, int &best_idx, int &best_splits)
 {
     const int kt_all = (K + 127) / 128;
@@ -1483,12 +1483,12 @@ void choose_config(int M, int N, int K, int &best_idx, int &best_splits)
                 break;
             const int64_t rounds = (tiles * s + 256 * c.wgs_per_cu - 1) / (256 * c.wgs_per_cu);
             const int steps = (kt_all + s - 1) / s;
-            const float fixed = c.bm == 256 ? 8000.f : 6000.f;   // fill and store of one workgroup
+            const float fixed = c.bm == 256 ? 6000.f : 6300.f;   // fill and store of one workgroup
             const float latency = (float)rounds * ((float)steps * c.step_cycles + fixed);
             const float throughput = (float)tiles * (float)s * (float)steps * c.step_cycles / 256.f + fixed;
             float cost = latency > throughput ? latency : throughput;
             if (s > 1)
-                cost += 4500.f + (float)s * (float)M * (float)N * 4.0f / 1350.f;
+                cost += 4500.f + (float)s * (float)M * (float)N * 4.0f / 950.f;
             if (cost < best) {
                 best = cost;
                 best_idx = i;
