@@ -23,3 +23,27 @@ def test_without_a_device_it_fails_loudly_instead_of_falling_back():
         return      # on a GPU box the benchmark itself is the check
     res = _run("--steps", "1", "--warmup", "0")
     assert res.returncode == 1 and "no HIP device" in res.stderr and res.stdout == ""
+
+
+def test_traffic_records_go_stale_with_their_source(tmp_path, monkeypatch):
+    """roofline.traffic comes from the committed counter summary only while the kernel's source
+    file still has the digest recorded there; otherwise the bench line says null."""
+    import hashlib
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("bench_under_test", os.path.join(ROOT, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    src = tmp_path / "kernel.hip"
+    src.write_text("__global__ void k() {}\n")
+    digest = hashlib.sha256(src.read_bytes()).hexdigest()[:16]
+    records = tmp_path / "traffic.md"
+    records.write_text("# summary\n\n"
+                       f"record: name=linear source={src} sha256={digest} bytes=168088496\n"
+                       f"record: name=quantize source={tmp_path / 'missing.hip'} sha256={digest} bytes=1\n")
+    monkeypatch.setattr(bench, "TRAFFIC_RECORDS", str(records))
+    assert bench.measured_traffic("linear") == 168088496.0
+    assert bench.measured_traffic("quantize") is None          # source file gone
+    assert bench.measured_traffic("dequantize") is None        # no record
+    src.write_text("__global__ void k() { }\n")                 # the kernel changed after the counter run
+    assert bench.measured_traffic("linear") is None
+
