@@ -1408,15 +1408,16 @@ struct TileConfig {
     int bm, bn;
     float step_cycles;  // one 128-byte K step of one workgroup: max(MFMA time, L2->LDS fill at ~40 B/clk)
     int wgs_per_cu;     // workgroups that fit a compute unit's LDS together
+    float busy_chip;    // factor on step_cycles when the whole chip runs such steps at once
 };
 constexpr TileConfig kTileConfigs[] = {
-    {32, 64, 441.f, 1}, {32, 128, 600.f, 2},
-    {64, 64, 432.f, 2},   // four stages
-    {64, 128, 611.f, 2},
-    {128, 64, 576.f, 1},  // four stages
-    {128, 128, 1050.f, 2},
-    {128, 128, 665.f, 1},  // four stages, eight waves: alone on its compute unit, for launches of one round
-    {256, 256, 2200.f, 1}};
+    {32, 64, 357.f, 1, 1.2f}, {32, 128, 540.f, 2, 0.8f},
+    {64, 64, 410.f, 2, 1.03f},   // four stages
+    {64, 128, 594.f, 2, 0.88f},
+    {128, 64, 554.f, 1, 0.8f},  // four stages
+    {128, 128, 1050.f, 2, 0.84f},
+    {128, 128, 593.f, 1, 1.05f},  // four stages, eight waves: alone on its compute unit, for launches of one round
+    {256, 256, 2200.f, 1, 1.0f}};
 constexpr int kNumTileConfigs = 8;
 
 // The epilogue addresses a tile's elements as a 32-bit offset (row in tile x N
@@ -1448,7 +1449,7 @@ int launch_config(int idx, const GemmArgs &g, int splits, hipStream_t st)
 // Picks the tile and the number of K ranges that minimise a simple cost
 // model, the larger of
 //   latency:    rounds of workgroups over the resident slots x K steps per workgroup x step cost
-//   throughput: all K steps of all workgroups x step cost / 256 compute units
+//   throughput: all K steps of all workgroups x step cost x busy-chip factor / 256 compute units
 // plus, for split K, the extra launch and the pass over the partial sums.
 // The constants were fitted (random search, least mean log regret) to two
 // exhaustive timing sweeps of every tile and split count over 72 shapes - one
@@ -1457,8 +1458,9 @@ int launch_config(int idx, const GemmArgs &g, int splits, hipStream_t st)
 // every launch streams them from HBM, since which tile wins can depend on that
 // (160x14336x4096: 64x128 tiles take 20.5 us cached and 30.5 us from HBM,
 // 128x128 tiles 22.6 and 25.4) - the shapes of the decode and MLP-chain
-// workloads weighted six-fold.  Mean regret 1.2 % cached and 0.7 % from HBM,
-// worst 13 % (192x8192x8192 and 6144x6144x2048 cached).
+// workloads weighted six-fold, plus 15 shapes of 8192 / 10240 / 28672 / 57344
+// columns from HBM.  Mean regret 1.2 % cached and 0.7 % from HBM, worst 14 %
+// (192x8192x8192 cached, 512x8192x28672 from HBM).
 void choose_config(int M, int N, int K, int &best_idx, int &best_splits)
 {
     const int kt_all = (K + 127) / 128;
@@ -1483,12 +1485,12 @@ void choose_config(int M, int N, int K, int &best_idx, int &best_splits)
                 break;
             const int64_t rounds = (tiles * s + 256 * c.wgs_per_cu - 1) / (256 * c.wgs_per_cu);
             const int steps = (kt_all + s - 1) / s;
-            const float fixed = c.bm == 256 ? 6000.f : 6300.f;   // fill and store of one workgroup
+            const float fixed = c.bm == 256 ? 4000.f : 6000.f;   // fill and store of one workgroup
             const float latency = (float)rounds * ((float)steps * c.step_cycles + fixed);
-            const float throughput = (float)tiles * (float)s * (float)steps * c.step_cycles / 256.f + fixed;
+            const float throughput = (float)tiles * (float)s * (float)steps * c.step_cycles * c.busy_chip / 256.f + fixed;
             float cost = latency > throughput ? latency : throughput;
             if (s > 1)
-                cost += 4500.f + (float)s * (float)M * (float)N * 4.0f / 950.f;
+                cost += 4500.f + (float)s * (float)M * (float)N * 4.0f / 1218.f;
             if (cost < best) {
                 best = cost;
                 best_idx = i;
