@@ -72,6 +72,8 @@ int vtl_hip_free(void *dptr);
 int vtl_hip_memcpy_h2d(void *dst_device, const void *src_host, size_t bytes);
 int vtl_hip_memcpy_d2h(void *dst_host, const void *src_device, size_t bytes);
 int vtl_hip_memcpy_d2d(void *dst_device, const void *src_device, size_t bytes);
+/* Byte fill on the current stream, any alignment and size; done by a kernel,
+ * so a caller's stream capture records a kernel node, not a memset node. */
 int vtl_hip_memset(void *dst_device, int byte_value, size_t bytes);
 
 /* Wait for everything enqueued on the current stream. */

@@ -60,6 +60,19 @@ def test_memset_and_device_to_device_copy(hip):
     b.release()
 
 
+@pytest.mark.parametrize("offset,size", [(0, 4096), (3, 1), (5, 10), (13, 1001), (1, 15), (16, 16), (7, 65537)])
+def test_memset_any_alignment_and_size_leaves_neighbours_alone(hip, offset, size):
+    buf = raw_device_buffer(70000)
+    h2d(buf.ptr, np.full(70000, 0x11, np.uint8))
+    capi.call("vtl_hip_memset", buf.ptr + offset, 0xC3, size)
+    capi.call("vtl_hip_sync")
+    got = d2h(buf.ptr, 70000, np.uint8)
+    want = np.full(70000, 0x11, np.uint8)
+    want[offset:offset + size] = 0xC3
+    assert np.array_equal(got, want)
+    buf.release()
+
+
 def test_events_time_a_kernel(hip):
     e0, e1 = C.c_void_p(), C.c_void_p()
     capi.call("vtl_hip_event_create", C.byref(e0))

@@ -6,6 +6,7 @@
 #include <string.h>
 
 #include <atomic>
+#include <mutex>
 
 #include "common.hpp"
 
@@ -38,9 +39,11 @@ int check_launch(const char *kernel_name)
 
 static Tuning g_tuning;
 static std::atomic<bool> g_tuning_read{false};
+static std::mutex g_tuning_mutex;
 
 static void read_tuning()
 {
+    std::lock_guard<std::mutex> lock(g_tuning_mutex);  // two first callers at once: one reads, the other waits
     Tuning t;
     auto flag = [](const char *name) { return getenv(name) != nullptr; };
     auto number = [](const char *name, int unset) {
@@ -184,6 +187,20 @@ void *library_workspace(size_t bytes, int slot)
     return buf[dev];
 }
 
+// Byte fill as a kernel (a memset node recorded into a caller's graph is avoided this way):
+// bytes up to the first 16-byte boundary, 16-byte vectors, remaining bytes.
+__global__ __launch_bounds__(256) void fill_bytes_kernel(unsigned char *p, unsigned word, size_t head, size_t nvec,
+                                                         size_t tail)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < nvec)
+        reinterpret_cast<uint4 *>(p + head)[i] = make_uint4(word, word, word, word);
+    if (i < head)
+        p[i] = (unsigned char)word;
+    if (i < tail)
+        p[head + nvec * 16 + i] = (unsigned char)word;
+}
+
 }  // namespace vtlhip
 
 using namespace vtlhip;
@@ -290,8 +307,18 @@ int vtl_hip_memset(void *dst_device, int byte_value, size_t bytes)
         return VTL_HIP_OK;
     if (!dst_device)
         return VTL_HIP_ERR_INVALID_ARG;
-    VTL_HIP_TRY(hipMemsetAsync(dst_device, byte_value, bytes, current_stream()));
-    return VTL_HIP_OK;
+    unsigned char *p = static_cast<unsigned char *>(dst_device);
+    size_t head = (16 - (reinterpret_cast<uintptr_t>(p) & 15)) & 15;
+    if (head > bytes)
+        head = bytes;
+    const size_t nvec = (bytes - head) >> 4, tail = (bytes - head) & 15;
+    const size_t blocks = ((nvec > 16 ? nvec : 16) + 255) / 256;
+    if (blocks > 0x7fffffffULL)
+        return VTL_HIP_ERR_UNSUPPORTED;
+    const unsigned word = 0x01010101u * (unsigned)(byte_value & 0xff);
+    hipLaunchKernelGGL(fill_bytes_kernel, dim3((unsigned)blocks), dim3(256), 0, current_stream(), p, word, head, nvec,
+                       tail);
+    return check_launch("fill_bytes_kernel");
 }
 
 int vtl_hip_sync(void)
