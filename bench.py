@@ -106,9 +106,137 @@ class Timer:
                 "note": "launches separated by an event record each: includes that gap, unlike kernel_us"}
 
 
-def bench_linear(timer: Timer, steps: int, warmup: int, cpu: bool):
+class PowerClockSampler:
+    """Samples the card's shader clock (one reading per XCD), socket power and the
+    power-throttle residency counter from a thread while the main thread keeps the GPU busy.
+    Readings come from the amdsmi Python binding of the ROCm image (the driver's gpu_metrics
+    table, which the firmware refreshes ONCE A SECOND: a load has to last a few seconds for
+    two or three fresh readings), or, when that is not importable, from the amdgpu hwmon /
+    pp_dpm_sclk sysfs files.  Measurement aid of this script only."""
+
+    def __init__(self, hz: float = 20.0):
+        import threading
+        self.period = 1.0 / hz
+        self.samples = []
+        self._stop = threading.Event()
+        self._thread = None
+        self._handle = None
+        self._smi = None
+        self.source = None
+        try:
+            import amdsmi
+            if not PowerClockSampler._smi_ready:
+                amdsmi.amdsmi_init()
+                PowerClockSampler._smi_ready = True
+            self._handle = amdsmi.amdsmi_get_processor_handles()[0]
+            amdsmi.amdsmi_get_gpu_metrics_info(self._handle)
+            self._smi = amdsmi
+            self.source = "amdsmi gpu_metrics (refreshed once a second)"
+        except Exception:                      # noqa: BLE001 - any failure means: use sysfs
+            self._smi = None
+            import glob
+            hw = glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input")
+            self._power_file = hw[0] if hw else None
+            dpm = glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk")
+            self._sclk_file = dpm[0] if dpm else None
+            self.source = "sysfs hwmon power1_input + pp_dpm_sclk" if hw or dpm else None
+
+    _smi_ready = False
+
+    def _read(self):
+        if self._smi is not None:
+            m = self._smi.amdsmi_get_gpu_metrics_info(self._handle)
+            clks = [c for c in m.get("current_gfxclks", []) if isinstance(c, int) and 0 < c < 10000]
+            return {"t": time.perf_counter(), "sclk": clks, "power_w": m.get("current_socket_power"),
+                    "energy": m.get("energy_accumulator"), "ppt_acc": m.get("ppt_residency_acc"),
+                    "acc": m.get("accumulation_counter"), "fw_t": m.get("firmware_timestamp")}
+        rec = {"t": time.perf_counter(), "sclk": [], "power_w": None}
+        try:
+            if self._power_file:
+                rec["power_w"] = int(open(self._power_file).read()) / 1e6
+            if self._sclk_file:
+                for line in open(self._sclk_file).read().splitlines():
+                    if line.rstrip().endswith("*"):
+                        rec["sclk"] = [int(line.split(":")[1].strip().split("M")[0])]
+        except (OSError, ValueError):
+            pass
+        return rec
+
+    def __enter__(self):
+        import threading
+        self.samples = []
+        self._stop.clear()
+        if self.source is None:
+            return self
+
+        def loop():
+            while not self._stop.is_set():
+                try:
+                    self.samples.append(self._read())
+                except Exception:              # noqa: BLE001
+                    pass
+                self._stop.wait(self.period)
+        self._thread = threading.Thread(target=loop, daemon=True)
+        self._thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop.set()
+        if self._thread:
+            self._thread.join()
+        return False
+
+    def summary(self, skip_s: float = 1.05):
+        """Means over the distinct readings taken later than skip_s after the start (a reading
+        describes the second before it, and the clock settles over the first tens of
+        milliseconds of load)."""
+        if not self.samples:
+            return {"source": self.source, "readings": 0}
+        t0 = self.samples[0]["t"]
+        distinct, seen = [], None
+        for x in self.samples:
+            key = (x.get("fw_t"), x.get("energy"), tuple(x["sclk"]), x.get("power_w"))
+            if key != seen:
+                distinct.append(x)
+                seen = key
+        if self._smi is not None:
+            distinct = distinct[1:]            # the first one was refreshed before the load began
+        ss = [x for x in distinct if x["t"] - t0 >= skip_s]
+        if not ss:
+            return {"source": self.source, "readings": 0,
+                    "note": "load too short for a fresh reading (raise --load-seconds)"}
+        clk = [np.mean(x["sclk"]) for x in ss if x["sclk"]]
+        per_xcd = [x["sclk"] for x in ss if x["sclk"]]
+        pw = [x["power_w"] for x in ss if isinstance(x.get("power_w"), (int, float))]
+        out = {"source": self.source, "readings": len(ss),
+               "sclk_mhz_mean": float(np.mean(clk)) if clk else None,
+               "sclk_mhz_per_xcd_min": float(np.min(per_xcd)) if per_xcd else None,
+               "sclk_mhz_per_xcd_max": float(np.max(per_xcd)) if per_xcd else None,
+               "power_w_mean": float(np.mean(pw)) if pw else None}
+        a, b = ss[0], ss[-1]
+        ints = lambda k: isinstance(a.get(k), int) and isinstance(b.get(k), int)   # noqa: E731
+        if len(ss) >= 2 and ints("energy") and ints("fw_t") and b["fw_t"] > a["fw_t"]:
+            # energy accumulator in units of 2^-16 J, firmware timestamp in units of 10 ns
+            out["power_w_from_energy_counter"] = ((b["energy"] - a["energy"]) * 15.259e-6 /
+                                                  ((b["fw_t"] - a["fw_t"]) * 1e-8))
+        if len(ss) >= 2 and ints("ppt_acc") and ints("acc") and b["acc"] > a["acc"]:
+            out["power_throttle_residency"] = (b["ppt_acc"] - a["ppt_acc"]) / (b["acc"] - a["acc"])
+        return out
+
+    def idle(self):
+        try:
+            r = self._read() if self.source else None
+        except Exception:                      # noqa: BLE001
+            r = None
+        return None if r is None else {"sclk_mhz": float(np.mean(r["sclk"])) if r["sclk"] else None,
+                                       "power_w": r.get("power_w")}
+
+
+def bench_linear(timer: Timer, steps: int, warmup: int, cpu: bool, load_s: float = 3.2, operands: str = "config"):
     m = n = k = 4096
     a, bt, sa, sb, bias = workloads.square_int8_gemm(m, n, k)
+    if operands == "zeros":       # diagnostic: the same launch without the data-dependent power draw
+        a, bt = np.zeros_like(a), np.zeros_like(bt)
     A, B = HipTensor.from_host(a), HipTensor.from_host(bt)
     SA, SB, BIAS = HipTensor.from_host(sa), HipTensor.from_host(sb), HipTensor.from_host(bias)
     Y = HipTensor.empty([m, n], np.float32)
@@ -122,8 +250,20 @@ def bench_linear(timer: Timer, steps: int, warmup: int, cpu: bool):
     ops = 2.0 * m * n * k
     kernel_ms = dev_ms / steps
     per_launch = timer.each(step, steps)
+    # shader clock and socket power while the same launch runs back to back for about load_s
+    # seconds (timed by its own event pair; not part of `value`)
+    under_load = None
+    if load_s > 0:
+        sampler = PowerClockSampler()
+        idle = sampler.idle()
+        n_load = max(steps, int(load_s / (kernel_ms * 1e-3)))
+        with sampler:
+            _, load_ms = timer.run(step, n_load)
+        under_load = sampler.summary()
+        under_load.update({"launches": n_load, "kernel_us": load_ms / n_load * 1e3, "idle_before": idle})
     res = {
         "per_launch": per_launch,
+        "under_load": under_load,
         "ms_per_step": wall * 1e3 / steps,
         "tops": ops / (wall / steps) / 1e12,
         "roofline": {"kernel": "gemm_i8_dma_kernel<256,256,128,2,2,4,f32 epilogue>", "bound": "mfma",
@@ -291,20 +431,19 @@ def bench_other_configs(timer: Timer, steps: int, warmup: int, cpu: bool = False
 
 
 def _other_decode_chain(timer: Timer, timed, out, parts, decode_cached: bool):
-    from vtl_amd.storage import HipStorage
-    rng = np.random.Generator(np.random.Philox(3))
     if "decode" in parts:
-        _bench_decode(timed, out, rng, decode_cached)
+        _bench_decode(timed, out, decode_cached)
     if "chain" in parts:
-        _bench_chain(timed, out, rng)
+        _bench_chain(timed, out)
     return out
 
 
-def _bench_decode(timed, out, rng, decode_cached: bool):
+def _bench_decode(timed, out, decode_cached: bool):
     from vtl_amd.storage import HipStorage
-    # configs[3]: K=4096, N=14336, M in {1,8,32,128}
+    # configs[3]: K=4096, N=14336, M in {1,8,32,128}; the tensors of workloads.decode_linear
+    # (seed 3), the ones the parity tests and the golden fixtures use
     k, n = 4096, 14336
-    W = HipTensor.from_host(rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02))
+    W = HipTensor.from_host(workloads.decode_linear(1, k, n)[1])
     Wq, Sw = W.quantize_i8(0)                      # one scale per output channel
     W.release()
     # The 58.7 MB of codes stay in the 256 MB last-level cache from one launch to the next.
@@ -315,7 +454,7 @@ def _bench_decode(timed, out, rng, decode_cached: bool):
         capi.call("vtl_hip_memcpy_d2d", c.ptr, Wq.ptr, n * k)
     dec = {}
     for m in (1, 8, 32, 128):
-        X = HipTensor.from_host(rng.standard_normal((m, k), dtype=np.float32))
+        X = HipTensor.from_host(workloads.decode_linear_activations(m, k))
         Y = HipTensor.empty([m, n], np.float32)
         need = int(capi.lib().vtl_hip_linear_f32_dynquant_workspace(m, k))
         ws = HipStorage.empty(need, np.uint8)
@@ -350,18 +489,20 @@ def _bench_decode(timed, out, rng, decode_cached: bool):
 
 
 
-def _bench_chain(timed, out, rng):
-    # configs[4]: 256x4096 -> 11008 -> ReLU -> 4096 -> ReLU -> 1024, device-resident chain
+def _bench_chain(timed, out):
+    # configs[4]: 256x4096 -> 11008 -> ReLU -> 4096 -> ReLU -> 1024, device-resident chain; the
+    # tensors of workloads.mlp_chain (seed 4), the ones the parity tests and the golden fixtures use
     dims, m = (4096, 11008, 4096, 1024), 256
+    x_host, ws_host = workloads.mlp_chain(m, dims)
     Ws, Ss = [], []
     for i in range(3):                             # Xavier-uniform f32 weights, one scale per output channel
-        bound = np.float32(np.sqrt(6.0 / (dims[i] + dims[i + 1])))
-        W = HipTensor.from_host((rng.random((dims[i + 1], dims[i]), dtype=np.float32) * 2 - 1) * bound)
+        W = HipTensor.from_host(ws_host[i])
         wq, sw = W.quantize_i8(0)
         W.release()
         Ws.append(wq)
         Ss.append(sw)
-    X = HipTensor.from_host(rng.standard_normal((m, dims[0]), dtype=np.float32))
+    del ws_host
+    X = HipTensor.from_host(x_host)
     # activations travel as per-token int8 codes + row scales: the first layer's input is
     # quantized, every hidden layer hands codes to the next (epilogue, ReLU and requantization
     # in one pass over the int32 sums), the last one writes f32
@@ -487,40 +628,104 @@ def bench_copy_calibration(timer: Timer, steps: int, warmup: int):
             "kernel_us": dev_ms / steps * 1e3, "GB/s": gbps}
 
 
-def bench_mfma_only(timer: Timer):
-    """What the matrix cores alone sustain: a probe kernel (a small library of its own, built
-    beside the product library and loaded only here) runs nothing but the
-    int8 MFMA of the matmul kernels, once on constant operands and once on uniformly random
-    ones (the operand distribution of configs[2]), each for a few tens of milliseconds so
-    that the clock has settled.  The random-operand figure is the ceiling that the power
+def bench_mfma_only(timer: Timer, load_s: float = 2.3):
+    """What the matrix cores alone sustain: probe kernels (a small library of its own, built
+    beside the product library and loaded only here) run nothing but the int8 MFMA of the
+    matmul kernels, on constant operands and on uniformly random ones (the operand
+    distribution of configs[2]), each for about load_s seconds while shader clock and socket
+    power are sampled.  Two loops: `fixed` re-uses 4 + 4 operand registers, `rotating` walks
+    through 32 + 32 register-resident fragments so that every instruction sees fresh operands,
+    like a matmul kernel's k-steps.  The random-operand figure is the ceiling that the power
     limit leaves to any int8 kernel on such data; the Linear's fraction of it is reported
     next to its fraction of the nominal peak."""
     from vtl_amd import build as vb
     if not os.path.exists(vb.BENCH_PROBE_PATH):
         vb.build_lib()
-    probe = C.CDLL(vb.BENCH_PROBE_PATH).vtl_bench_probe_mfma_i8
-    probe.restype, probe.argtypes = C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
+    lib = C.CDLL(vb.BENCH_PROBE_PATH)
     stream = C.c_void_p()
     capi.call("vtl_hip_get_stream", C.byref(stream))
     rng = np.random.Generator(np.random.Philox(2))
     sink = HipTensor.empty([4], np.int32)
     out = {}
-    iters = 4000
-    ops = 1024.0 * 4 * 16 * iters * 65536.0
-    for label, host in (("constant_operands", np.full(32768, 1, np.int8)),
-                        ("uniform_random_operands", rng.integers(-127, 128, 32768, dtype=np.int8))):
-        buf = HipTensor.from_host(host)
+    nbytes = 256 * 1024
+    hosts = (("constant_operands", np.full(nbytes, 1, np.int8)),
+             ("uniform_random_operands", rng.integers(-127, 128, nbytes, dtype=np.int8)))
+    for loop, sym, per_iter, iters in (("fixed", "vtl_bench_probe_mfma_i8", 16, 4000),
+                                       ("rotating", "vtl_bench_probe_mfma_i8_rotating", 64, 1000)):
+        probe = getattr(lib, sym)
+        probe.restype, probe.argtypes = C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
+        ops = 1024.0 * 4 * per_iter * iters * 65536.0
+        for label, host in hosts:
+            buf = HipTensor.from_host(host)
 
-        def step():
-            if probe(buf.ptr, iters, sink.ptr, stream) != 0:
-                raise RuntimeError("vtl_bench_probe_mfma_i8 failed")
-        for _ in range(4):
-            step()
-        _, dev_ms = timer.run(step, 8)
-        out[label] = {"TOP/s": ops / (dev_ms / 8 * 1e-3) / 1e12, "us_per_launch": dev_ms / 8 * 1e3}
-        buf.release()
+            def step():
+                if probe(buf.ptr, iters, sink.ptr, stream) != 0:
+                    raise RuntimeError(sym + " failed")
+            for _ in range(4):
+                step()
+            _, dev_ms = timer.run(step, 8)
+            n = max(8, int(load_s / (dev_ms / 8 * 1e-3)))
+            sampler = PowerClockSampler()
+            with sampler:
+                _, dev_ms = timer.run(step, n)
+            rec = {"TOP/s": ops / (dev_ms / n * 1e-3) / 1e12, "us_per_launch": dev_ms / n * 1e3,
+                   "under_load": sampler.summary()}
+            if loop == "fixed":
+                out[label] = rec
+            else:
+                out.setdefault("rotating_operand_registers", {})[label] = rec
+            buf.release()
     sink.release()
     return out
+
+
+def _vendor_yardstick_child(steps: int, warmup: int) -> int:
+    """Body of the child process behind bench_vendor_yardstick(): prints one JSON object."""
+    try:
+        import torch
+        if not torch.cuda.is_available():
+            print(json.dumps({"error": "torch sees no GPU"}))
+            return 0
+        a, bt, _, _, _ = workloads.square_int8_gemm()
+        A = torch.from_numpy(a).cuda()
+        Bt = torch.from_numpy(bt).cuda()
+        B = Bt.t()                                   # K x N view of the weights as stored [N,K]
+        for _ in range(warmup):
+            c = torch._int_mm(A, B)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            c = torch._int_mm(A, B)
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) / steps * 1e3
+        want = a[:8].astype(np.int64) @ bt.astype(np.int64).T
+        ok = bool(np.array_equal(c[:8].cpu().numpy().astype(np.int64), want))
+        print(json.dumps({
+            "what": "torch._int_mm(A, Wq^T) -> int32 (PyTorch-ROCm hands it to hipBLASLt), the operands of "
+                    "configs[2], int32 sums out (the same 64 MiB as the Linear's f32 result), no scale/bias epilogue; "
+                    "a yard-stick, not part of the product and never `value`",
+            "us": us, "TOP/s": 2.0 * 4096 ** 3 / us / 1e6, "frac_of_peak": 2.0 * 4096 ** 3 / us / 1e6 / PEAK_INT8_TOPS,
+            "steps": steps, "warmup": warmup, "sums_match_numpy_on_8_rows": ok, "torch": torch.__version__}))
+    except Exception as e:                            # noqa: BLE001 - a yard-stick must never fail the bench
+        print(json.dumps({"error": repr(e)[:200]}))
+    return 0
+
+
+def bench_vendor_yardstick(steps: int, warmup: int):
+    """The vendor library's int8 matmul on the same operands, timed in a child process (PyTorch
+    brings its own HIP runtime, which is kept out of the process that loads libvtlhip.so).
+    None when the child gives no answer."""
+    import subprocess
+    try:
+        res = subprocess.run([sys.executable, os.path.abspath(__file__), "--vendor-yardstick-child",
+                              "--steps", str(steps), "--warmup", str(warmup)],
+                             stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True, timeout=240)
+        lines = [l for l in res.stdout.splitlines() if l.startswith("{")]
+        return json.loads(lines[-1]) if lines else None
+    except Exception as e:                            # noqa: BLE001
+        return {"error": repr(e)[:200]}
 
 
 def main() -> int:
@@ -533,6 +738,14 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only", choices=["all", "linear", "quant", "copy", "full", "other", "mfma", "decode", "chain"],
                     default="all")
+    ap.add_argument("--linear-operands", choices=["config", "zeros"], default="config",
+                    help="zeros: time the Linear on all-zero int8 operands (a diagnostic, says so in the line)")
+    ap.add_argument("--load-seconds", type=float, default=3.2,
+                    help="length of the back-to-back loops during which clock and power are sampled (0: none)")
+    ap.add_argument("--no-probe", action="store_true", help="skip the MFMA-only probe loops (profiling runs)")
+    ap.add_argument("--vendor-yardstick-child", action="store_true", help=argparse.SUPPRESS)
+    ap.add_argument("--no-vendor-yardstick", action="store_true",
+                    help="skip the torch._int_mm timing printed beside the Linear")
     ap.add_argument("--decode-from-hbm-only", action="store_true",
                     help="with --only decode: skip the launches that re-read the same weights (profiling)")
     args = ap.parse_args()
@@ -540,6 +753,8 @@ def main() -> int:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 "
               "(sharding across GPUs is a design note only; nothing multi-GPU is built)", file=sys.stderr)
         return 2
+    if args.vendor_yardstick_child:
+        return _vendor_yardstick_child(args.steps, args.warmup)
     if capi.device_count() < 1:
         print("bench.py: no HIP device visible", file=sys.stderr)
         return 1
@@ -561,10 +776,10 @@ def main() -> int:
                                                                not args.decode_from_hbm_only)}))
         return 0
     if args.only == "mfma":
-        print(json.dumps({"mfma_only": bench_mfma_only(timer)}))
+        print(json.dumps({"mfma_only": bench_mfma_only(timer, max(args.load_seconds, 0.05))}))
         return 0
 
-    lin = bench_linear(timer, args.steps, args.warmup, cpu) if args.only in ("all", "linear") else None
+    lin = bench_linear(timer, args.steps, args.warmup, cpu, args.load_seconds, args.linear_operands) if args.only in ("all", "linear") else None
     qd = bench_quant(timer, args.steps, args.warmup, cpu) if args.only in ("all", "quant") else None
 
     line = {
@@ -580,6 +795,8 @@ def main() -> int:
                                 "[16384,16384], seed 1") if lin else qd["quantize"]["config"]["workload"],
                    "device": name, "compute_units": cus, "clock_mhz": mhz},
     }
+    if lin and args.linear_operands != "config":
+        line["diagnostic"] = "all-zero int8 operands, NOT the configs[2] workload"
     if lin:
         line["roofline"] = lin["roofline"]
         line["per_launch"] = lin["per_launch"]
@@ -595,9 +812,17 @@ def main() -> int:
         line["quantize"] = qd["quantize"]
         line["dequantize"] = qd["dequantize"]
     if lin:
-        line["mfma_only"] = bench_mfma_only(timer)
-        line["roofline"]["frac_of_mfma_only_rate_on_these_operands"] = (
-            line["roofline"]["achieved"] / line["mfma_only"]["uniform_random_operands"]["TOP/s"])
+        ul = lin.get("under_load") or {}
+        line["roofline"]["sclk_mhz_under_load"] = ul.get("sclk_mhz_mean")
+        line["roofline"]["power_w"] = ul.get("power_w_mean")
+        line["under_load"] = ul
+        if not args.no_probe:
+            line["mfma_only"] = bench_mfma_only(timer, max(args.load_seconds * 0.72, 0.05))
+            ceiling = max(line["mfma_only"]["uniform_random_operands"]["TOP/s"],
+                          line["mfma_only"]["rotating_operand_registers"]["uniform_random_operands"]["TOP/s"])
+            line["roofline"]["frac_of_mfma_only_rate_on_these_operands"] = line["roofline"]["achieved"] / ceiling
+        if not args.no_vendor_yardstick:
+            line["vendor_int8_mm"] = bench_vendor_yardstick(args.steps, args.warmup)
     if args.only == "all":
         line["other_configs"] = bench_other_configs(timer, args.steps, args.warmup, cpu)
         line["full_precision"] = bench_full_precision(timer, args.steps, args.warmup)

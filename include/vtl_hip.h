@@ -34,8 +34,12 @@
  *     i.e. issue them on one stream (or order the streams yourself).  The
  *     buffers grow on demand, which waits for the whole device; while the
  *     current stream is being captured into a graph a call that would have to
- *     grow one returns VTL_HIP_ERR_UNSUPPORTED instead (run it once before
- *     capturing).
+ *     grow one returns VTL_HIP_ERR_UNSUPPORTED instead (pass a workspace of
+ *     your own where the entry point takes one, use
+ *     vtl_hip_linear_f32_dynquant_noalloc, or run the call once before
+ *     capturing).  A buffer that a recorded graph uses is never freed: when a
+ *     later call needs a larger one it gets a new buffer and the old one stays
+ *     allocated until the process ends, so replays of the graph stay valid.
  */
 #ifndef VTL_HIP_H
 #define VTL_HIP_H
@@ -248,7 +252,8 @@ const char *vtl_hip_last_error(void);
 const char *vtl_hip_version(void);
 /* The library reads its tuning switches (environment variables VTL_HIP_*, used
  * by tests and tuning runs only) once, at the first call that looks at them;
- * this reads them again. */
+ * this reads them again.  A test and tuning aid, not part of the path: launches
+ * that run on other threads meanwhile see the old switches or the new ones. */
 int vtl_hip_reload_env(void);
 
 #ifdef __cplusplus

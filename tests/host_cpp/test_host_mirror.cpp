@@ -139,18 +139,48 @@ int main(int argc, char **argv)
             vtl_ref_linear_f32_dynquant(xin.data(), wq.data(), sw.data(), bf.data(), out.data(), m, n, k, relu, 1);
             return out;
         };
-        auto y1 = s.linear_forward_f32(x, M, K, w, N, b, &w, nullptr);
+        // frozen parameters (inference): quantized once, the copy is kept
+        auto y1 = s.linear_forward_f32(x, M, K, w, N, b, &w, nullptr, true);
         void *ws_first = s.workspace.ptr;
         void *codes_first = s.layers[0].w_q.data.ptr;
-        auto y1b = s.linear_forward_f32(x, M, K, w, N, b, &w, nullptr);
+        auto y1b = s.linear_forward_f32(x, M, K, w, N, b, &w, nullptr, true);
         CHECK(s.layers.size() == 1 && s.quantize_count == 1);          // quantized once
         CHECK(s.workspace.ptr == ws_first && s.layers[0].w_q.data.ptr == codes_first);
         CHECK(y1 == y1b && y1 == ref_linear(x, M, K, w, N, b, false));
-        // an optimizer step replaces the weight tensor: same slot, new codes
+        // Adam assigns a new weight tensor: same slot, new codes
         for (auto &v : w1b) v = -v;
-        auto y1c = s.linear_forward_f32(x, M, K, w1b, N, b, &w, nullptr);
+        auto y1c = s.linear_forward_f32(x, M, K, w1b, N, b, &w, nullptr, true);
         CHECK(s.layers.size() == 1 && s.quantize_count == 2);
         CHECK(y1c == ref_linear(x, M, K, w1b, N, b, false));
+        // SGD-style step: the SAME tensor updated in place (nn/internal/optimizers.v:6-12).  A
+        // training forward (not frozen) quantizes every time and always sees the new values ...
+        {
+            std::vector<float> wt = w, bt = b;
+            const int before = s.quantize_count;
+            auto t0 = s.linear_forward_f32(x, M, K, wt, N, bt, &wt, nullptr);
+            CHECK(t0 == ref_linear(x, M, K, wt, N, bt, false));
+            for (size_t i = 0; i < wt.size(); i++) wt[i] -= 0.1f * w1b[i];
+            for (auto &v : bt) v -= 0.05f;
+            auto t1 = s.linear_forward_f32(x, M, K, wt, N, bt, &wt, nullptr);
+            CHECK(t1 == ref_linear(x, M, K, wt, N, bt, false));
+            CHECK(s.quantize_count == before + 2);
+            // ... a frozen forward does not trust the copy a training forward made ...
+            for (size_t i = 0; i < wt.size(); i++) wt[i] += 0.3f * w1b[i];
+            auto t2 = s.linear_forward_f32(x, M, K, wt, N, bt, &wt, nullptr, true);
+            CHECK(t2 == ref_linear(x, M, K, wt, N, bt, false) && s.quantize_count == before + 3);
+            auto t3 = s.linear_forward_f32(x, M, K, wt, N, bt, &wt, nullptr, true);
+            CHECK(t3 == t2 && s.quantize_count == before + 3);
+            // ... and notices an in-place edit of frozen parameters by their fingerprint
+            for (auto &v : wt) v *= 0.5f;
+            auto t4 = s.linear_forward_f32(x, M, K, wt, N, bt, &wt, nullptr, true);
+            CHECK(t4 == ref_linear(x, M, K, wt, N, bt, false) && s.quantize_count == before + 4);
+            for (auto &v : bt) v = 0.25f;
+            auto t5 = s.linear_forward_f32(x, M, K, wt, N, bt, &wt, nullptr, true);
+            CHECK(t5 == ref_linear(x, M, K, wt, N, bt, false));
+            s.invalidate(&wt);
+            auto t6 = s.linear_forward_f32(x, M, K, wt, N, bt, &wt, nullptr, true);
+            CHECK(t6 == t5 && s.quantize_count == before + 5);
+        }
         // Linear -> ReLU -> Linear with the activation staying on the device
         auto h = s.linear_forward_f32(x, M, K, w, N, b, &w, nullptr);
         CHECK(s.has_pending);
@@ -162,7 +192,7 @@ int main(int argc, char **argv)
         auto r_dev = s.take_pending();
         auto out = s.linear_forward_f32(r, M, N, w2, O, b2, &w2, &r_dev);
         CHECK(out == ref_linear(r_ref, M, N, w2, O, b2, false));
-        CHECK(s.layers.size() == 2);
+        CHECK(s.layers.size() == 3);
         // the whole chain with int8 hand-off equals the layer-by-layer result bit for bit
         auto chain = s.mlp_forward_i8(x, M, {&w, &w2}, {&b, &b2}, {K, N, O}, {true, false});
         auto h_relu = ref_linear(x, M, K, w, N, b, true);

@@ -12,7 +12,7 @@ from helpers import CPU_THREADS, KAT, dev, rel_err, raw_device_buffer, h2d, d2h
 from vtl_amd import capi, workloads
 from vtl_amd.tensor import HipTensor, gemm_i8_hip, linear_i8_hip
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("guard_bands")]
 
 F32_REL_TOL = 1e-5   # tolerance stated for dequantized f32 outputs
 

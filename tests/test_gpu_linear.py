@@ -9,7 +9,7 @@ from vtl_amd import (PER_CHANNEL, PER_TENSOR, HipSession, QuantLinearLayer, Sequ
                      linear_forward_hip_f32, workloads)
 from vtl_amd.tensor import HipTensor, linear_f32_dynquant_hip
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("guard_bands")]
 
 F32_REL_TOL = 1e-5
 
@@ -145,15 +145,63 @@ def test_weight_cache_follows_parameter_replacement(hip):
     w1 = rng.standard_normal((8, 64)).astype(np.float32)
     w2 = rng.standard_normal((8, 64)).astype(np.float32)
     x = rng.standard_normal((3, 64)).astype(np.float32)
-    layer = QuantLinearLayer(w1)
+    layer = QuantLinearLayer(w1, requires_grad=False)
     y1 = layer.forward(x)
     first = layer.quantized()
-    assert layer.quantized() is first                 # reused while the parameter is the same object
-    layer.weights = w2                                # optimizers assign a new tensor (adam.v:115,136)
+    assert layer.quantized() is first                 # frozen parameter, same object: reused
+    layer.weights = w2                                # Adam assigns a new tensor (adam.v:115,136)
     y2 = layer.forward(x)
     assert layer.quantized() is not first
     assert np.array_equal(y1, _oracle_linear(x, w1, None, PER_CHANNEL))
     assert np.array_equal(y2, _oracle_linear(x, w2, None, PER_CHANNEL))
+    layer.release()
+
+
+def test_weight_cache_sees_in_place_optimizer_steps(hip):
+    """SGD, AdaGrad, AdamW and RMSProp update `v.value` in place (nn/optimizers/sgd.v:46-53 ->
+    nn/internal/optimizers.v:6-12): the tensor object stays the same while its contents change.
+    A trainable layer therefore quantizes its parameters on every forward; a frozen one keeps
+    them, and still notices an in-place edit through the content fingerprint."""
+    rng = np.random.default_rng(7)
+    w = rng.standard_normal((8, 64)).astype(np.float32)
+    b = rng.standard_normal((1, 8)).astype(np.float32)
+    g = rng.standard_normal((8, 64)).astype(np.float32)
+    x = rng.standard_normal((3, 64)).astype(np.float32)
+    layer = QuantLinearLayer(w, b)                    # requires_grad, like every reference Variable
+    y0 = layer.forward(x)
+    assert np.array_equal(y0, _oracle_linear(x, w.copy(), b.reshape(-1), PER_CHANNEL))
+    for step in range(2):                             # sgd_optimize: value.set(i, val - lr * grad)
+        layer.weights -= np.float32(0.1) * g
+        layer.bias -= np.float32(0.05)
+        assert layer.weights is w and np.shares_memory(layer.bias, b)   # same tensors, new contents
+        y = layer.forward(x)
+        assert np.array_equal(y, _oracle_linear(x, w.copy(), b.reshape(-1), PER_CHANNEL)), step
+    assert layer.quantize_count == 3                  # every training forward re-quantized
+    # inference: the copy made under no_grad is kept ...
+    n0 = layer.quantize_count
+    y_a = layer.forward(x, no_grad=True)
+    y_b = layer.forward(x, no_grad=True)
+    assert layer.quantize_count == n0 + 1 and np.array_equal(y_a, y_b)
+    # ... a training forward in between never trusts it, nor is its own copy trusted afterwards
+    layer.forward(x)
+    layer.weights += np.float32(0.25) * g
+    y_c = layer.forward(x, no_grad=True)
+    assert np.array_equal(y_c, _oracle_linear(x, w.copy(), b.reshape(-1), PER_CHANNEL))
+    # ... and an in-place edit of frozen parameters (a checkpoint loaded into the same tensors)
+    layer.requires_grad = False
+    layer.forward(x)
+    n1 = layer.quantize_count
+    layer.forward(x)
+    assert layer.quantize_count == n1
+    w[...] = rng.standard_normal((8, 64)).astype(np.float32)
+    y_d = layer.forward(x)
+    assert layer.quantize_count == n1 + 1
+    assert np.array_equal(y_d, _oracle_linear(x, w.copy(), b.reshape(-1), PER_CHANNEL))
+    b[...] = 0.5                                      # the bias alone
+    y_e = layer.forward(x)
+    assert np.array_equal(y_e, _oracle_linear(x, w.copy(), b.reshape(-1), PER_CHANNEL))
+    layer.invalidate()
+    assert np.array_equal(layer.forward(x), y_e) and layer.quantize_count == n1 + 3
     layer.release()
 
 

@@ -12,7 +12,7 @@ import oracle
 from helpers import CPU_THREADS, dev
 from vtl_amd.tensor import HipTensor, gemm_i8_hip, linear_i8_hip, linear_f32_dynquant_hip
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("guard_bands")]
 
 
 def _draw_shape(rng):

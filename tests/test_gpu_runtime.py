@@ -186,16 +186,36 @@ def test_entry_points_capture_into_a_hip_graph(hip):
 def test_mfma_probe_runs_and_leaves_its_sink_alone(hip):
     """The measurement aid behind bench.py's `mfma_only` figures: launches, finishes, and
     never writes its sink (the sums it keeps alive cannot reach the sentinel)."""
-    ops = HipTensor.from_host(np.random.default_rng(0).integers(-127, 128, 32768, dtype=np.int8))
+    ops = HipTensor.from_host(np.random.default_rng(0).integers(-127, 128, 256 * 1024, dtype=np.int8))
     sink = HipTensor.from_host(np.array([-7, 0, 0, 0], np.int32))
     from vtl_amd import build as vb
     assert os.path.exists(vb.BENCH_PROBE_PATH), "libvtlbenchprobe.so is not built"
-    probe = C.CDLL(vb.BENCH_PROBE_PATH).vtl_bench_probe_mfma_i8
-    probe.restype, probe.argtypes = C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
-    assert probe(ops.ptr, 3, sink.ptr, None) == 0
-    assert probe(ops.ptr, 0, sink.ptr, None) == 0
-    capi.call("vtl_hip_sync")
-    assert sink.cpu()[0] == -7
-    assert probe(ops.ptr + 1, 3, sink.ptr, None) == 1
+    for sym in ("vtl_bench_probe_mfma_i8", "vtl_bench_probe_mfma_i8_rotating"):
+        probe = getattr(C.CDLL(vb.BENCH_PROBE_PATH), sym)
+        probe.restype, probe.argtypes = C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
+        assert probe(ops.ptr, 3, sink.ptr, None) == 0
+        assert probe(ops.ptr, 0, sink.ptr, None) == 0
+        capi.call("vtl_hip_sync")
+        assert sink.cpu()[0] == -7
+        assert probe(ops.ptr + 1, 3, sink.ptr, None) == 1
     ops.release()
     sink.release()
+
+
+def test_guard_bands_notice_a_write_past_either_end(hip, guard_bands):
+    """The out-of-bounds check of the ragged-shape parity tests, checked itself: a byte written
+    just before or just past a buffer (inside the guarded allocation, so nothing faults) is
+    reported when the buffer is released; an untouched buffer is not."""
+    clean = HipTensor.from_host(np.arange(100, dtype=np.float32))
+    assert np.array_equal(clean.cpu(), np.arange(100, dtype=np.float32))
+    clean.release()
+    assert guard_bands == []
+    past = HipTensor.empty([3, 7], np.int8)
+    capi.call("vtl_hip_memset", past.ptr + 21, 0, 1)
+    past.release()
+    assert len(guard_bands) == 1 and "after the buffer" in guard_bands[0] and "offset 0 " in guard_bands[0]
+    before = HipTensor.empty([5], np.int32)
+    capi.call("vtl_hip_memset", before.ptr - 2, 7, 1)
+    before.release()
+    assert len(guard_bands) == 2 and "before the buffer" in guard_bands[1] and "offset -2 " in guard_bands[1]
+    guard_bands.clear()

@@ -27,7 +27,11 @@ bool launch_copy(void *dst, const void *src, size_t bytes, hipStream_t st);
 // slot 2: int8 operands repacked to a row length the fast kernels take),
 // grown on demand and kept until the process ends.  Kernels enqueued on the
 // current stream may use a slot until the next call that asks for it; nullptr
-// when the allocation fails.
+// when the allocation fails.  While the current stream records a graph a slot
+// is handed out only if it is already large enough (growing would free and
+// allocate), and a buffer handed out then is never freed afterwards, because
+// replays of the graph keep using its address: a later, larger request gets a
+// new buffer and the old one stays allocated.
 void *library_workspace(size_t bytes, int slot = 0);
 // Why the last library_workspace() call of this thread returned nullptr
 // (VTL_HIP_ERR_OUT_OF_MEMORY, or VTL_HIP_ERR_UNSUPPORTED when the request does

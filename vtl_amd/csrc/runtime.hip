@@ -37,41 +37,48 @@ int check_launch(const char *kernel_name)
     return VTL_HIP_OK;
 }
 
-static Tuning g_tuning;
-static std::atomic<bool> g_tuning_read{false};
+// The switches are published as an immutable snapshot behind an atomic pointer:
+// a launch that reads them while vtl_hip_reload_env() runs on another thread
+// sees the old snapshot or the new one, never a half-written struct.  Replaced
+// snapshots are not freed (a reader may still hold one; a reload is a test and
+// tuning aid, a few dozen bytes each).
+static std::atomic<const Tuning *> g_tuning{nullptr};
 static std::mutex g_tuning_mutex;
 
-static void read_tuning()
+static const Tuning *read_tuning(bool force)
 {
     std::lock_guard<std::mutex> lock(g_tuning_mutex);  // two first callers at once: one reads, the other waits
-    Tuning t;
+    if (!force) {
+        if (const Tuning *seen = g_tuning.load(std::memory_order_acquire))
+            return seen;
+    }
+    Tuning *t = new Tuning;
     auto flag = [](const char *name) { return getenv(name) != nullptr; };
     auto number = [](const char *name, int unset) {
         const char *v = getenv(name);
         return v ? atoi(v) : unset;
     };
-    t.no_gemv = flag("VTL_HIP_NO_GEMV");
-    t.gemv_rows = number("VTL_HIP_GEMV_ROWS", -1);
-    t.gemm_small = number("VTL_HIP_GEMM_SMALL", -1);
+    t->no_gemv = flag("VTL_HIP_NO_GEMV");
+    t->gemv_rows = number("VTL_HIP_GEMV_ROWS", -1);
+    t->gemm_small = number("VTL_HIP_GEMM_SMALL", -1);
     if (const char *v = getenv("VTL_HIP_GEMM_CONFIG")) {
         int idx = -1, splits = 1;
         // a value that does not parse still takes the launch off the special-case kernels
-        t.gemm_config = (sscanf(v, "%d,%d", &idx, &splits) >= 1 && idx >= 0) ? idx : 1 << 30;
-        t.gemm_splits = splits;
+        t->gemm_config = (sscanf(v, "%d,%d", &idx, &splits) >= 1 && idx >= 0) ? idx : 1 << 30;
+        t->gemm_splits = splits;
     }
-    t.no_fused_requant = flag("VTL_HIP_NO_FUSED_REQUANT");
-    t.no_fused_decode = flag("VTL_HIP_NO_FUSED_DECODE");
-    t.matmul_tile = number("VTL_HIP_MATMUL_TILE", 0);
-    t.matmul_splits = number("VTL_HIP_MATMUL_SPLITS", -1);
-    g_tuning = t;
-    g_tuning_read.store(true, std::memory_order_release);
+    t->no_fused_requant = flag("VTL_HIP_NO_FUSED_REQUANT");
+    t->no_fused_decode = flag("VTL_HIP_NO_FUSED_DECODE");
+    t->matmul_tile = number("VTL_HIP_MATMUL_TILE", 0);
+    t->matmul_splits = number("VTL_HIP_MATMUL_SPLITS", -1);
+    g_tuning.store(t, std::memory_order_release);
+    return t;
 }
 
 const Tuning &tuning()
 {
-    if (!g_tuning_read.load(std::memory_order_acquire))
-        read_tuning();
-    return g_tuning;
+    const Tuning *t = g_tuning.load(std::memory_order_acquire);
+    return t ? *t : *read_tuning(false);
 }
 
 // ---- scratch for callers that cannot allocate --------------------------------
@@ -130,6 +137,7 @@ void *library_workspace(size_t bytes, int slot)
 {
     static void *bufs[3][kMaxDevices] = {};
     static size_t caps[3][kMaxDevices] = {};
+    static bool captured[3][kMaxDevices] = {};   // the buffer's address is baked into a recorded graph
     g_workspace_status = VTL_HIP_OK;
     if (slot < 0 || slot > 2) {
         g_workspace_status = VTL_HIP_ERR_INVALID_ARG;
@@ -150,31 +158,39 @@ void *library_workspace(size_t bytes, int slot)
     }
     void **buf = bufs[slot];
     size_t *cap = caps[slot];
+    bool *in_graph = captured[slot];
     const int dev = current_device();
     if (dev < 0) {
         g_workspace_status = VTL_HIP_ERR_NO_DEVICE;
         return nullptr;
     }
+    // Is the current stream recording a graph?  A query that fails counts as "yes": the
+    // cautious answer, since growing frees and allocates and neither may happen then.
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(current_stream(), &capturing) != hipSuccess) {
+        (void)hipGetLastError();
+        capturing = hipStreamCaptureStatusActive;
+    }
+    const bool recording = capturing != hipStreamCaptureStatusNone;
     if (bytes > cap[dev]) {
-        // Growing frees the old buffer, which kernels of any stream may still use, and allocates:
-        // neither is possible while the current stream records a graph.
-        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-        if (hipStreamIsCapturing(current_stream(), &capturing) != hipSuccess)
-            (void)hipGetLastError();
-        if (capturing != hipStreamCaptureStatusNone) {
+        if (recording) {
             snprintf(g_last_error, sizeof(g_last_error),
-                     "library scratch would have to grow to %zu bytes during a stream capture: run the call once "
-                     "before capturing",
+                     "library scratch would have to grow to %zu bytes during a stream capture: pass a workspace "
+                     "of your own, use the entry point that allocates nothing, or run the call once before "
+                     "capturing",
                      bytes);
             g_workspace_status = VTL_HIP_ERR_UNSUPPORTED;
             return nullptr;
         }
-        if (buf[dev]) {
+        if (buf[dev] && !in_graph[dev]) {
             (void)hipDeviceSynchronize();   // every stream: the buffer is shared by all of them
             (void)hipFree(buf[dev]);
-            buf[dev] = nullptr;
-            cap[dev] = 0;
         }
+        // A buffer that a recorded graph refers to is never freed: replays of that graph keep
+        // writing to it.  It stays allocated until the process ends and a new one takes its place.
+        buf[dev] = nullptr;
+        cap[dev] = 0;
+        in_graph[dev] = false;
         const size_t want = bytes < (size_t(32) << 20) ? (size_t(32) << 20) : bytes;
         if (hipMalloc(&buf[dev], want) != hipSuccess) {
             (void)hipGetLastError();
@@ -184,6 +200,8 @@ void *library_workspace(size_t bytes, int slot)
         }
         cap[dev] = want;
     }
+    if (recording)
+        in_graph[dev] = true;
     return buf[dev];
 }
 
@@ -393,7 +411,7 @@ const char *vtl_hip_last_error(void) { return g_last_error; }
 
 int vtl_hip_reload_env(void)
 {
-    read_tuning();
+    (void)read_tuning(true);
     return VTL_HIP_OK;
 }
 

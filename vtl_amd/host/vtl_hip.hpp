@@ -12,6 +12,7 @@
 
 #include <cstdint>
 #include <cstdlib>
+#include <cstring>
 #include <stdexcept>
 #include <string>
 #include <type_traits>
@@ -364,15 +365,49 @@ inline std::vector<std::vector<float>> linear_backward_hip_f32(const std::vector
     return {dx.cpu(), dw.cpu(), bias_needs_grad ? db.to_array() : std::vector<float>((size_t)n, 0.0f)};
 }
 
+// Cheap fingerprint of a parameter tensor's contents: FNV-1a over the bit patterns of
+// up to 64 elements at even strides plus the last one, and the element count.
+inline uint64_t content_fingerprint(const std::vector<float> &t)
+{
+    const size_t n = t.size();
+    uint64_t h = 0xcbf29ce484222325ULL ^ (uint64_t)n;
+    auto mix = [&](float v) {
+        uint32_t bits;
+        memcpy(&bits, &v, sizeof bits);
+        h = (h ^ bits) * 0x100000001b3ULL;
+    };
+    if (n) {
+        const size_t step = n / 64 ? n / 64 : 1;
+        size_t taken = 0;
+        for (size_t i = 0; i < n && taken < 64; i += step, taken++)
+            mix(t[i]);
+        mix(t[n - 1]);
+    }
+    return h;
+}
+
 // `HipSession` (autograd_hip/hip_session_d_hip.v): per-Context device state of the
 // INT8 path - the staging buffer of the activation quantization, the int8 weights of
-// every layer that ran through it (quantized once; `slot` names the layer, `source`
-// the weight tensor the codes were made from, so a replaced tensor is re-quantized)
-// and the f32 rows the last layer left on the device for the next one.
+// every layer that ran through it (`slot` names the layer) and the f32 rows the last
+// layer left on the device for the next one.
+//
+// When the device copy of a layer's parameters is re-used: most of the reference's
+// optimizers update `v.value` IN PLACE (SGD: nn/optimizers/sgd.v:46-53 ->
+// nn/internal/optimizers.v:6-12 `value.set`; adagrad.v:60, adamw.v:95, rmsprop.v:81),
+// only Adam assigns a new tensor (adam.v:115,136), so the identity of the weight tensor
+// says nothing about its contents.  A forward that is not `frozen` (the Context is not
+// no_grad and the weight Variable requires grad) uploads and quantizes the parameters
+// again, as the reference's own device chain uploads them on every forward
+// (autograd_cuda/device_session_gpu_d_cuda.v:107).  A `frozen` forward re-uses the copy
+// only if it was made by a frozen forward from the same tensors and their content
+// fingerprints are unchanged (an in-place checkpoint load is seen that way);
+// invalidate() drops a copy explicitly.
 class HipSession {
 public:
     struct QuantizedWeights {
         const void *slot = nullptr, *source = nullptr, *bias_source = nullptr;
+        uint64_t fingerprint = 0, bias_fingerprint = 0;
+        bool frozen = false;
         HipTensor<int8_t> w_q;
         HipTensor<float> sw;
         HipStorage<float> bias;
@@ -404,9 +439,16 @@ public:
             workspace = HipStorage<uint8_t>(need);
         return workspace;
     }
-    // `weights` / `bias` are the host tensors' storage; their addresses are the cache keys
+    // drops the device copy of one layer (slot) or of all layers (null)
+    void invalidate(const void *slot = nullptr)
+    {
+        for (auto &l : layers)
+            if (!slot || l.slot == slot)
+                l.source = l.bias_source = nullptr;
+    }
+    // `weights` / `bias` are the host tensors' storage
     QuantizedWeights &quantized(const void *slot, const std::vector<float> &weights, int n, int k,
-                                const std::vector<float> &bias)
+                                const std::vector<float> &bias, bool frozen)
     {
         QuantizedWeights *q = nullptr;
         for (auto &l : layers)
@@ -417,27 +459,33 @@ public:
             q = &layers.back();
             q->slot = slot;
         }
-        if (q->source != (const void *)&weights || !q->w_q.data.ptr) {
+        const bool trust = frozen && q->frozen;
+        const uint64_t fp = content_fingerprint(weights), bfp = content_fingerprint(bias);
+        if (!trust || q->source != (const void *)&weights || q->fingerprint != fp || !q->w_q.data.ptr) {
             auto w_dev = HipTensor<float>::from_host(weights, {n, k});
             auto qs = quantize_i8(w_dev, 0);
             q->w_q = std::move(qs.first);
             q->sw = std::move(qs.second);
             q->source = &weights;
+            q->fingerprint = fp;
             quantize_count++;
         }
-        if (q->bias_source != (const void *)&bias || !q->bias.ptr) {
+        if (!trust || q->bias_source != (const void *)&bias || q->bias_fingerprint != bfp || !q->bias.ptr) {
             q->bias = HipStorage<float>::from_cpu(bias);
             q->bias_source = &bias;
+            q->bias_fingerprint = bfp;
         }
+        q->frozen = frozen;
         return *q;
     }
-    // `(mut s HipSession) linear_forward_f32(x, weights, bias, slot, input_gpu) !&vtl.Tensor[f32]`:
+    // `(mut s HipSession) linear_forward_f32(x, weights, bias, slot, input_gpu, frozen) !&vtl.Tensor[f32]`:
     // host rows out; the device rows stay pending for the next layer.  `input_gpu` is a
-    // device activation taken from the previous layer (take_pending) or null.
+    // device activation taken from the previous layer (take_pending) or null; `frozen`
+    // says that no optimizer can have touched the parameters (see the class comment).
     std::vector<float> linear_forward_f32(const std::vector<float> &x, int m, int k,
                                           const std::vector<float> &weights, int n,
                                           const std::vector<float> &bias, const void *slot,
-                                          HipTensor<float> *input_gpu)
+                                          HipTensor<float> *input_gpu, bool frozen = false)
     {
         if (!enabled)
             throw HipError("hip session disabled", VTL_HIP_ERR_NO_DEVICE);
@@ -445,7 +493,7 @@ public:
             throw std::invalid_argument("Invalid shapes for matrix multiplication");
         pending.release();
         has_pending = false;
-        QuantizedWeights &q = quantized(slot, weights, n, k, bias);
+        QuantizedWeights &q = quantized(slot, weights, n, k, bias, frozen);
         const HipStorage<uint8_t> &ws = ensure_workspace(m, k);
         HipTensor<float> uploaded;
         const HipTensor<float> *x_dev = input_gpu;
@@ -484,6 +532,7 @@ public:
     }
     // `mlp_forward_i8(x, weights, biases, relu_after, slots)`: the whole chain on the device,
     // int8 codes handed from layer to layer, f32 rows of the last layer back to the host.
+    // An inference call: the parameters count as frozen.
     std::vector<float> mlp_forward_i8(const std::vector<float> &x, int m,
                                       const std::vector<const std::vector<float> *> &weights,
                                       const std::vector<const std::vector<float> *> &biases,
@@ -498,10 +547,10 @@ public:
         auto cur = quantize_i8(x_dev, 0);
         x_dev.release();
         for (size_t i = 0; i + 1 < nl; i++) {
-            QuantizedWeights &q = quantized(weights[i], *weights[i], dims[i + 1], dims[i], *biases[i]);
+            QuantizedWeights &q = quantized(weights[i], *weights[i], dims[i + 1], dims[i], *biases[i], true);
             cur = linear_i8_requant_hip(cur.first, cur.second, q.w_q, q.sw, &q.bias, relu_after[i]);
         }
-        QuantizedWeights &q = quantized(weights[nl - 1], *weights[nl - 1], dims[nl], dims[nl - 1], *biases[nl - 1]);
+        QuantizedWeights &q = quantized(weights[nl - 1], *weights[nl - 1], dims[nl], dims[nl - 1], *biases[nl - 1], true);
         return linear_i8_hip(cur.first, cur.second, q.w_q, q.sw, &q.bias, relu_after[nl - 1]).cpu();
     }
 };

@@ -88,19 +88,42 @@ class HipSession:
         self._bufs.clear()
 
 
+def content_fingerprint(t: np.ndarray) -> int:
+    """Cheap fingerprint of a parameter tensor's contents: FNV-1a over the bit patterns of
+    up to 64 elements at even strides plus the last one, and the element count.  It is
+    the second line of defence of the weight cache (the first is the frozen rule of
+    QuantLinearLayer.quantized): an in-place edit of a frozen parameter - a checkpoint
+    loaded into the same tensor, a manual `set` - changes it with near certainty when
+    the edit touches most elements, as every optimizer step and every load does."""
+    flat = np.ascontiguousarray(t).reshape(-1).view(np.uint32 if t.dtype.itemsize == 4 else np.uint64)
+    n = flat.size
+    h = 0xcbf29ce484222325 ^ n
+    if n:
+        step = max(1, n // 64)
+        for v in list(flat[::step][:64]) + [flat[n - 1]]:
+            h = ((h ^ int(v)) * 0x100000001b3) & 0xffffffffffffffff
+    return h
+
+
 class QuantizedWeights:
-    """Device-resident int8 weights of one Linear layer, derived once from the
-    f32 parameter (the reference's optimizers assign a new tensor each step,
-    nn/optimizers/adam.v:115,136, so the cache is keyed on the array object)."""
+    """Device-resident int8 weights of one Linear layer, derived from the f32
+    parameter.  `source` / `bias_source` are the host tensors the device copies
+    were made from, `fingerprint` / `bias_fingerprint` their content fingerprints at
+    that moment and `frozen` whether the parameters were frozen then (see
+    QuantLinearLayer.quantized for the rule that decides re-use)."""
 
     def __init__(self, weights: np.ndarray, bias: np.ndarray | None, mode: str,
-                 params: HipParams | None = None):
+                 params: HipParams | None = None, frozen: bool = False):
         if weights.ndim != 2:
             raise ValueError("Matrix expected")
         if mode not in (PER_TENSOR, PER_CHANNEL):
             raise ValueError(f"unknown quantization mode {mode!r}")
         self.mode = mode
         self.source = weights
+        self.bias_source = bias
+        self.frozen = frozen
+        self.fingerprint = content_fingerprint(weights)
+        self.bias_fingerprint = None if bias is None else content_fingerprint(np.asarray(bias))
         self.out_features, self.in_features = weights.shape
         w_dev = HipTensor.from_host(np.asarray(weights, np.float32), params)
         try:
@@ -174,10 +197,23 @@ def _linear_host_roundtrip(x, weights, bias, mode) -> np.ndarray:
 class QuantLinearLayer:
     """`LinearLayer[f32]` (nn/layers/linear.v:17-74) whose forward runs on the
     INT8 HIP path.  Parameters stay on the host as f32 (as in the reference);
-    the int8 copy is derived state, rebuilt when `weights` is replaced."""
+    the int8 copy on the device is derived state.
+
+    `requires_grad` mirrors the flag of the layer's weight Variable
+    (autograd/variable.v:64, default true): while it is set an optimizer may
+    change the parameters between any two forwards, and most of the reference's
+    optimizers do so IN PLACE (SGD: nn/optimizers/sgd.v:46-53 ->
+    nn/internal/optimizers.v:6-12 `value.set`; likewise adagrad.v:60, adamw.v:95,
+    rmsprop.v:81), only Adam assigns a new tensor (adam.v:115,136).  So the
+    tensor's identity says nothing about its contents, and a trainable layer
+    uploads and quantizes its parameters on every forward, as the reference's
+    own device chain uploads them on every forward
+    (autograd_cuda/device_session_gpu_d_cuda.v:107).  The codes are kept from
+    one forward to the next only for frozen parameters (requires_grad false, or
+    a forward under no_grad)."""
 
     def __init__(self, weights: np.ndarray, bias: np.ndarray | None = None, mode: str = PER_CHANNEL,
-                 params: HipParams | None = None):
+                 params: HipParams | None = None, requires_grad: bool = True):
         weights = np.asarray(weights, np.float32)
         if weights.ndim != 2:
             raise ValueError("Matrix expected")
@@ -186,6 +222,8 @@ class QuantLinearLayer:
                      else np.asarray(bias, np.float32).reshape(1, -1))  # [1, out]
         self.mode = mode
         self.params = params or HipParams()
+        self.requires_grad = requires_grad
+        self.quantize_count = 0      # how often the parameters were uploaded and quantized (tests)
         self._cache: QuantizedWeights | None = None
 
     def output_shape(self):
@@ -194,24 +232,42 @@ class QuantLinearLayer:
     def variables(self):
         return [self.weights, self.bias]
 
-    def quantized(self) -> QuantizedWeights:
-        if self._cache is None or self._cache.source is not self.weights:
-            if self._cache is not None:
-                self._cache.release()
-            self._cache = QuantizedWeights(self.weights, self.bias, self.mode, self.params)
+    def invalidate(self) -> None:
+        """Drops the device copy: the next forward uploads and quantizes again.  For
+        callers that edit a frozen parameter in place."""
+        if self._cache is not None:
+            self._cache.release()
+            self._cache = None
+
+    def quantized(self, no_grad: bool = False) -> QuantizedWeights:
+        """The layer's int8 weights for one forward.  Re-used from the previous forward only
+        when ALL of these hold: the parameters are frozen now (`requires_grad` false, or this
+        forward runs under `no_grad`) and were frozen when the copy was made, `weights` and
+        `bias` are still the same tensor objects, and their content fingerprints have not
+        changed.  Otherwise the parameters are uploaded and quantized again."""
+        frozen = no_grad or not self.requires_grad
+        c = self._cache
+        fresh = (c is not None and frozen and c.frozen and c.source is self.weights
+                 and c.bias_source is self.bias and c.fingerprint == content_fingerprint(self.weights)
+                 and c.bias_fingerprint == content_fingerprint(self.bias))
+        if not fresh:
+            if c is not None:
+                c.release()
+            self._cache = QuantizedWeights(self.weights, self.bias, self.mode, self.params, frozen=frozen)
+            self.quantize_count += 1
         return self._cache
 
     def forward_device(self, x: HipTensor, relu: bool = False,
-                       session: HipSession | None = None) -> HipTensor:
-        return linear_forward_hip_i8_device(x, self.quantized(), relu=relu, session=session)
+                       session: HipSession | None = None, no_grad: bool = False) -> HipTensor:
+        return linear_forward_hip_i8_device(x, self.quantized(no_grad), relu=relu, session=session)
 
-    def forward(self, x: np.ndarray) -> np.ndarray:
+    def forward(self, x: np.ndarray, no_grad: bool = False) -> np.ndarray:
         x = np.asarray(x, np.float32)
         if x.ndim != 2:
             raise ValueError("Matrix expected")
         x_dev = HipTensor.from_host(x, self.params)
         try:
-            y = self.forward_device(x_dev)
+            y = self.forward_device(x_dev, no_grad=no_grad)
             try:
                 return y.cpu()
             finally:

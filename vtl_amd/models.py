@@ -51,7 +51,10 @@ class Sequential:
         self.layers.append(("relu",))
         return self
 
-    def forward(self, x: np.ndarray) -> np.ndarray:
+    def forward(self, x: np.ndarray, no_grad: bool = False) -> np.ndarray:
+        """`no_grad` is the Context's flag (autograd/context.v:19-21): under it the layers'
+        quantized weights are kept from one forward to the next, otherwise every trainable
+        layer uploads and quantizes its parameters again (QuantLinearLayer.quantized)."""
         x = np.asarray(x, np.float32)
         if x.ndim != 2:
             raise ValueError("Matrix expected")
@@ -67,7 +70,7 @@ class Sequential:
                     j = i + (2 if fuse else 1)
                     feeds_linear = self.mode == PER_CHANNEL and j < n and self.layers[j][0] == "linear"
                     if cur_q is None and not feeds_linear:
-                        nxt = layer.forward_device(cur, relu=fuse, session=self.session)
+                        nxt = layer.forward_device(cur, relu=fuse, session=self.session, no_grad=no_grad)
                         cur.release()
                         cur = nxt
                     else:
@@ -77,7 +80,7 @@ class Sequential:
                             cur_q = cur.quantize_i8(0)
                             cur.release()
                             cur = None
-                        qw = layer.quantized()
+                        qw = layer.quantized(no_grad)
                         if feeds_linear:
                             nxt_q = linear_i8_requant_hip(cur_q[0], cur_q[1], qw.w_q, qw.sw, qw.bias, relu=fuse)
                         else:

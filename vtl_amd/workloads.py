@@ -55,12 +55,17 @@ def square_int8_gemm(m: int = 4096, n: int = 4096, k: int = 4096, seed: int = 2)
     return a, bt, sa, sb, bias
 
 
+def decode_linear_activations(m: int, k: int = 4096, seed: int = 3) -> np.ndarray:
+    """Config 4's activations ~N(0,1) [m, k] alone (a stream of their own per m, so that the
+    weights do not depend on m)."""
+    return _rng(seed * 1000 + m).standard_normal((m, k), dtype=np.float32)
+
+
 def decode_linear(m: int, k: int = 4096, n: int = 14336, seed: int = 3):
     """Config 4: f32 weights ~N(0, 0.02) stored [n, k], activations ~N(0,1) [m, k]."""
     rng = _rng(seed)
     w = (rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02))
-    x = _rng(seed * 1000 + m).standard_normal((m, k), dtype=np.float32)
-    return x, w
+    return decode_linear_activations(m, k, seed), w
 
 
 def xavier_uniform(out_features: int, in_features: int, rng: np.random.Generator) -> np.ndarray:
