@@ -263,6 +263,40 @@ def test_few_token_kernel_and_its_alternatives(hip, mnk, rows_kernel, knobs):
         h.release()
 
 
+# the weight-streaming kernel on blocks of 32 activation rows x 32 weight rows (small outputs
+# with a long K, M > 32; also M <= 32 against few weight rows): whole and ragged blocks in both
+# directions, one block, one round of workgroups and two, every row-count class of a block
+# (<= 8, <= 16, <= 32 rows in the last block), K of one chunk per wave and of uneven shares
+ROW_BLOCK_SHAPES = [(256, 1024, 4096), (250, 1000, 4096), (33, 4096, 2048), (64, 64, 4096), (100, 2500, 1024),
+                    (40, 31, 1024), (65, 33, 1280), (72, 96, 2304), (48, 50, 11008), (300, 40, 768),
+                    (16, 1024, 4096), (5, 500, 2048), (32, 64, 1024), (1000, 32, 1024)]
+
+
+@pytest.mark.parametrize("waves", ["4", "2", "0", None])
+@pytest.mark.parametrize("mnk", ROW_BLOCK_SHAPES)
+def test_row_block_weight_streaming_kernel_and_its_alternatives(hip, mnk, waves, knobs):
+    """VTL_HIP_SKINNY_TILED=1 forces the kernel (with VTL_HIP_SKINNY_WAVES waves a workgroup),
+    0 keeps it off, unset is the library's own choice: same int32 sums, same f32 rows."""
+    if waves is None:
+        knobs.delenv("VTL_HIP_SKINNY_TILED", raising=False)
+    elif waves == "0":
+        knobs.setenv("VTL_HIP_SKINNY_TILED", "0")
+    else:
+        knobs.setenv("VTL_HIP_SKINNY_WAVES", waves)
+        knobs.setenv("VTL_HIP_SKINNY_TILED", "1")
+    m, n, k = mnk
+    a, bt, sa, sb, bias = workloads.square_int8_gemm(m, n, k, seed=m * 37 + n * 11 + k)
+    ref = oracle.gemm_i8_i32(a, bt, threads=CPU_THREADS)
+    assert np.array_equal(_gemm(a, bt), ref)
+    A, B, dsa, dsb, dbias = dev(a), dev(bt), dev(sa), dev(sb), dev(bias)
+    for relu, b_dev, b_host in ((True, dbias, bias), (False, None, None)):
+        y = linear_i8_hip(A, dsa, B, dsb, b_dev, relu=relu)
+        assert np.array_equal(y.cpu(), oracle.epilogue(ref, sa, sb, b_host, relu=relu))
+        y.release()
+    for h in (A, B, dsa, dsb, dbias):
+        h.release()
+
+
 @pytest.mark.parametrize("k", [2432, 2448, 80])   # 19 K steps of 128; the same plus a 16-byte tail; one partial step
 def test_forced_split_k_is_exact(hip, knobs, k):
     """Every tile configuration with 1, 2, 3 and 8 K ranges gives the same int32 result

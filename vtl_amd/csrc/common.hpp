@@ -63,6 +63,8 @@ struct Tuning {
     int gemm_splits = 1;
     bool no_fused_requant = false;  // VTL_HIP_NO_FUSED_REQUANT: linear, then the row quantizer
     bool no_fused_decode = false;   // VTL_HIP_NO_FUSED_DECODE: quantizer launch in front of the linear
+    int skinny_tiled = -1;          // VTL_HIP_SKINNY_TILED: 1 / 0 force the 32x32-block weight-streaming kernel for M > 32
+    int skinny_waves = 4;           // VTL_HIP_SKINNY_WAVES: 2, 4 or 8 waves (K ranges) per workgroup there
     int matmul_tile = 0;            // VTL_HIP_MATMUL_TILE: 128 / 64 force the f64-accumulating tile
     int matmul_splits = -1;         // VTL_HIP_MATMUL_SPLITS: K ranges of the f64-accumulating matmul
 };

@@ -642,7 +642,9 @@ int launch_finalize_requant(const GemmArgs &g, hipStream_t st)
 
 // Weight-streaming kernel for M <= 32 (decode-shaped linear): bound by reading
 // the weight matrix once, so the design goal is bytes in flight and long
-// contiguous reads, not MFMA rate.  A workgroup owns 32 weight rows (128 KiB of
+// contiguous reads, not MFMA rate.  (With more activation rows grid.y walks
+// blocks of 32 of them: the form used for small outputs with a long K, see
+// skinny_blocks_waves.)  A workgroup owns 32 weight rows (128 KiB of
 // contiguous memory when K = 4096); its NWAVE waves split K between them and
 // each wave runs a PRIVATE software pipeline - its own LDS ring of STAGES
 // slots (32 rows x 256 bytes of Wq plus the activation rows that exist),
@@ -672,6 +674,7 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_skinny_kernel(const GemmArg
     const int M = g.M, N = g.N, K = g.K;
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int n0 = blockIdx.x * 32;
+    const int m0 = blockIdx.y * 32;   // more than 32 activation rows: one block of 32 per grid row
     char *ring = smem + w * (STAGES * SLOT);
 
     // K range of this wave, in 256-byte chunks
@@ -695,7 +698,7 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_skinny_kernel(const GemmArg
     for (int j = 0; j < XLOADS; j++) {
         const int row = lrow + 4 * j;
         const int lc = (lane & 15) ^ (row & 15);
-        px[j] = g.A + (int64_t)min(row, M - 1) * K + (int64_t)kc_begin * BK + lc * 16;
+        px[j] = g.A + (int64_t)min(m0 + row, M - 1) * K + (int64_t)kc_begin * BK + lc * 16;
     }
     auto issue = [&](int c, int st) {
         char *sw_ = ring + st * SLOT;
@@ -772,11 +775,12 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_skinny_kernel(const GemmArg
     __syncthreads();
     // 256 (m, 4 x n) items; 8 threads cover the 128-byte row segment of one m
     for (int item = tid; item < 256; item += 64 * NWAVE) {
-        const int m = item >> 3, nq = (item & 7) * 4;
-        v4i sum = *reinterpret_cast<const v4i *>(part + m * 32 + nq);
+        const int ml = item >> 3, nq = (item & 7) * 4;
+        v4i sum = *reinterpret_cast<const v4i *>(part + ml * 32 + nq);
 #pragma unroll
         for (int ww = 1; ww < NWAVE; ww++)
-            sum += *reinterpret_cast<const v4i *>(part + ww * 1024 + m * 32 + nq);
+            sum += *reinterpret_cast<const v4i *>(part + ww * 1024 + ml * 32 + nq);
+        const int m = m0 + ml;
         if (m >= M)
             continue;
         const int n = n0 + nq;
@@ -1240,14 +1244,18 @@ __global__ __launch_bounds__(256) void pad_rows_i8_kernel(const int8_t *__restri
     reinterpret_cast<unsigned *>(dst)[i] = w;
 }
 
-// Small products (a few dozen 32x32 output tiles): nothing is reused often
-// enough to stage, so each wave feeds the MFMA straight from global memory.
-// One workgroup per 32x32 tile; its four waves split the K steps and the
-// partial tiles meet in LDS.  Needs K % 16 == 0 and 16-byte aligned operands.
-template <bool F32OUT>
-__global__ __launch_bounds__(256) void gemm_i8_small_kernel(const GemmArgs g)
+// Small products (up to a few hundred 32x32 output tiles): nothing is reused
+// often enough to stage, so each wave feeds the MFMA straight from global memory.
+// One workgroup per 32x32 tile; its NW waves split the K steps (U steps of loads
+// in flight per wave) and the partial tiles meet in LDS.  With sixteen waves a
+// tile with K = 4096 is two rounds of loads per wave, so a product like
+// 256x1024x4096 (256 tiles, one per compute unit) is one launch whose length is
+// a couple of memory latencies, instead of a K-split launch plus the pass that
+// adds the partial sums.  Needs K % 16 == 0 and 16-byte aligned operands.
+template <bool F32OUT, int NW, int U>
+__global__ __launch_bounds__(64 * NW) void gemm_i8_small_kernel(const GemmArgs g)
 {
-    __shared__ int red[4][16][64];
+    __shared__ int red[NW][16][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int tiles_n = (g.N + 31) / 32;
     const int m0 = (int)(blockIdx.x / tiles_n) * 32, n0 = (int)(blockIdx.x % tiles_n) * 32;
@@ -1258,17 +1266,17 @@ __global__ __launch_bounds__(256) void gemm_i8_small_kernel(const GemmArgs g)
     const int8_t *__restrict__ ap = g.A + (int64_t)arow * g.K + 16 * half;
     const int8_t *__restrict__ bp = g.Bt + (int64_t)brow * g.K + 16 * half;
     const int steps = (g.K + 31) / 32;
-    const int per = (steps + 3) / 4;
+    const int per = (steps + NW - 1) / NW;
     const int t0 = wave * per, t1 = t0 + per < steps ? t0 + per : steps;
     v16i acc;
 #pragma unroll
     for (int i = 0; i < 16; ++i)
         acc[i] = 0;
     const v4i zero = {0, 0, 0, 0};
-    for (int t = t0; t < t1; t += 4) {   // four steps of loads in flight
-        v4i a[4], b[4];
+    for (int t = t0; t < t1; t += U) {   // U steps of loads in flight
+        v4i a[U], b[U];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < U; ++u) {
             const int k = 32 * (t + u);
             // K % 32 == 16: the upper half of the last step is empty
             const bool in = t + u < t1 && k + 16 * half < g.K;
@@ -1276,18 +1284,19 @@ __global__ __launch_bounds__(256) void gemm_i8_small_kernel(const GemmArgs g)
             b[u] = in ? *reinterpret_cast<const v4i *>(bp + k) : zero;
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
+        for (int u = 0; u < U; ++u)
             acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[u], b[u], acc, 0, 0, 0);
     }
 #pragma unroll
     for (int i = 0; i < 16; ++i)
         red[wave][i][lane] = acc[i];
     __syncthreads();
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int o = threadIdx.x + 256 * j;
+    for (int o = threadIdx.x; o < 1024; o += 64 * NW) {
         const int reg = o >> 6, l = o & 63;
-        const int sum = (red[0][reg][l] + red[1][reg][l]) + (red[2][reg][l] + red[3][reg][l]);
+        int sum = 0;
+#pragma unroll
+        for (int w = 0; w < NW; ++w)
+            sum += red[w][reg][l];
         // accumulator register reg of lane l: row 8 * (reg / 4) + 4 * (l / 32) + reg % 4, column l % 32
         const int m = m0 + 8 * (reg >> 2) + 4 * (l >> 5) + (reg & 3), n = n0 + (l & 31);
         if (m >= g.M || n >= g.N)
@@ -1507,22 +1516,62 @@ int launch_skinny_cfg(const GemmArgs &g, hipStream_t st)
     static_assert(lds >= NWAVE * 4096, "room for the partial tiles");
     static PerDevice<bool> done_flag;
     bool &done = done_flag.get();
-    const int blocks = (g.N + 31) / 32;
-    return launch_with_lds(linear_skinny_kernel<NWAVE, STAGES, XJ, F32OUT>, done, lds, blocks, 64 * NWAVE, g, st,
-                           "linear_skinny_kernel");
+    const dim3 grid((unsigned)((g.N + 31) / 32), (unsigned)((g.M + 31) / 32));
+    if (grid.y > 65535)
+        return VTL_HIP_ERR_UNSUPPORTED;
+    if (!done) {  // one host thread per device
+        VTL_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(linear_skinny_kernel<NWAVE, STAGES, XJ, F32OUT>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        done = true;
+    }
+    hipLaunchKernelGGL((linear_skinny_kernel<NWAVE, STAGES, XJ, F32OUT>), grid, dim3(64 * NWAVE), lds, st, g);
+    return check_launch("linear_skinny_kernel");
 }
 
+// nwave: K ranges (waves) per workgroup.  Two waves and two ring slots measured best for the
+// decode shapes (M <= 32 against thousands of weight rows): the small LDS footprint keeps every
+// workgroup of the grid resident at once, and that parallelism hides latency better than a
+// deeper ring per wave does.  Four waves are for grids of at most one workgroup per compute
+// unit, where the K split is the only parallelism left.
 template <bool F32OUT>
-int launch_skinny(const GemmArgs &g, hipStream_t st)
+int launch_skinny(const GemmArgs &g, int nwave, hipStream_t st)
 {
-    // Two waves and two ring slots per workgroup measured best: the small LDS
-    // footprint keeps every workgroup of the grid resident at once, and that
-    // parallelism hides latency better than a deeper ring per wave does.
+    if (nwave == 4) {
+        if (g.M <= 8)
+            return launch_skinny_cfg<4, 2, 1, F32OUT>(g, st);
+        if (g.M <= 16)
+            return launch_skinny_cfg<4, 2, 2, F32OUT>(g, st);
+        return launch_skinny_cfg<4, 2, 4, F32OUT>(g, st);
+    }
     if (g.M <= 8)
         return launch_skinny_cfg<2, 2, 1, F32OUT>(g, st);
     if (g.M <= 16)
         return launch_skinny_cfg<2, 2, 2, F32OUT>(g, st);
     return launch_skinny_cfg<2, 2, 4, F32OUT>(g, st);
+}
+
+// The weight-streaming kernel on blocks of 32 activation rows x 32 weight rows (grid.y walks
+// the row blocks) for small outputs with a long K: every block is a workgroup whose waves cut
+// K between them, so a product like 256x1024x4096 (256 blocks, one per compute unit) is one
+// launch of 6.1 us where the tile kernels need a K split and a second launch to fill the chip
+// (10.0 us); 33x4096x2048 4.9 against 8.1 us, 256x1024x11008 10.9 against 13.7 us.  Returns
+// the number of waves per workgroup (4: at most one round of workgroups, one per compute unit;
+// 2: up to two rounds of two per compute unit), or 0 where the tile kernels are as fast or
+// faster (short K: everything is launch-bound; more blocks: the tiles' operand reuse wins;
+// few blocks with a very long K: the tile kernels' finer K split wins).  Measured over
+// K = 256 ... 8192 and 4 ... 512 blocks.
+inline int skinny_blocks_waves(int M, int N, int K)
+{
+    if (tuning().skinny_tiled >= 0)   // 1 / 0 force the choice (tests, tuning)
+        return tuning().skinny_tiled != 0 ? tuning().skinny_waves : 0;
+    const int64_t blocks = (int64_t)((M + 31) / 32) * ((N + 31) / 32);
+    if (K < 1024)
+        return 0;
+    if (blocks <= 256)
+        return (K <= 4096 || blocks >= 96) ? 4 : 0;
+    if (blocks <= 512)
+        return K <= 4096 ? 2 : 0;
+    return 0;
 }
 
 // Waves of the single-token kernel's grid: no more than the chip holds at once, sixteen per
@@ -1653,6 +1702,19 @@ inline bool gemv_applies(const void *row, const void *w, int N, int K)
            !tuning().no_gemv;
 }
 
+// Where one workgroup per 32x32 tile, fed straight from global memory, beats the tile kernels:
+// few tiles and a short K (nothing to stage), and up to a chip's worth of tiles with a long K,
+// which the tile kernels could only fill the chip with by cutting K (a second launch).
+inline bool small_product_faster(int64_t t32, int K)
+{
+    return t32 <= 64 && K <= 2048;
+}
+inline int small_product_waves(int64_t t32, int K)
+{
+    (void)t32;
+    return K <= 2048 ? 4 : (K <= 4096 ? 8 : 16);
+}
+
 template <bool F32OUT>
 int launch_gemm(const GemmArgs &g_in, hipStream_t st)
 {
@@ -1696,11 +1758,25 @@ int launch_gemm(const GemmArgs &g_in, hipStream_t st)
     if (gemv_rows_applies(g.A, g.Bt, g.M, g.N, g.K) && gemv_rows_faster(g.M, g.N, g.K) && !config_set && !small_set)
         return launch_gemv_rows<false, F32OUT>(g, st);
     if (g.K % 256 == 0 && g.M <= 32 && g.N >= 2048 && !config_set)
-        return launch_skinny<F32OUT>(g, st);  // weight streaming: enough row blocks to fill the chip
+        return launch_skinny<F32OUT>(g, 2, st);  // weight streaming: enough row blocks to fill the chip
+    if (g.K % 256 == 0 && !config_set && !small_set) {
+        const int nwave = skinny_blocks_waves(g.M, g.N, g.K);
+        if (nwave)
+            return launch_skinny<F32OUT>(g, nwave == 2 ? 2 : 4, st);
+    }
     const int64_t t32 = (int64_t)((g.M + 31) / 32) * ((g.N + 31) / 32);
-    // VTL_HIP_GEMM_SMALL 1 / 0 forces the choice (tests, tuning)
-    if (small_set ? tn.gemm_small != 0 : (t32 <= 64 && g.K <= 2048)) {
-        hipLaunchKernelGGL((gemm_i8_small_kernel<F32OUT>), dim3((unsigned)t32), dim3(256), 0, st, g);
+    // VTL_HIP_GEMM_SMALL 1 / 0 forces the choice (tests, tuning); 4, 8, 16 also the number of waves
+    if (small_set ? tn.gemm_small != 0 : small_product_faster(t32, g.K)) {
+        if (t32 > 0x7fffffff)
+            return VTL_HIP_ERR_UNSUPPORTED;
+        const int nw = tn.gemm_small >= 4 ? tn.gemm_small : small_product_waves(t32, g.K);
+        const dim3 grid((unsigned)t32);
+        if (nw >= 16)
+            hipLaunchKernelGGL((gemm_i8_small_kernel<F32OUT, 16, 8>), grid, dim3(1024), 0, st, g);
+        else if (nw >= 8)
+            hipLaunchKernelGGL((gemm_i8_small_kernel<F32OUT, 8, 8>), grid, dim3(512), 0, st, g);
+        else
+            hipLaunchKernelGGL((gemm_i8_small_kernel<F32OUT, 4, 4>), grid, dim3(256), 0, st, g);
         return check_launch("gemm_i8_small_kernel");
     }
     int idx, splits;

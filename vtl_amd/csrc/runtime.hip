@@ -69,6 +69,8 @@ static const Tuning *read_tuning(bool force)
     }
     t->no_fused_requant = flag("VTL_HIP_NO_FUSED_REQUANT");
     t->no_fused_decode = flag("VTL_HIP_NO_FUSED_DECODE");
+    t->skinny_tiled = number("VTL_HIP_SKINNY_TILED", -1);
+    t->skinny_waves = number("VTL_HIP_SKINNY_WAVES", 4);
     t->matmul_tile = number("VTL_HIP_MATMUL_TILE", 0);
     t->matmul_splits = number("VTL_HIP_MATMUL_SPLITS", -1);
     g_tuning.store(t, std::memory_order_release);
