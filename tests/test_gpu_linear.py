@@ -69,14 +69,19 @@ def test_decode_linear_config(hip, m):
 # size class (N <= 1024 ... 16384), and the shapes that fall back to linear + row quantizer
 # (few rows, N % 4 != 0, N > 16384, K % 16 != 0)
 REQUANT_SHAPES = [(256, 1024, 4096), (256, 4096, 11008), (256, 11008, 4096), (100, 1200, 1360), (64, 2048, 512),
+                  (130, 4100, 640), (200, 8200, 272), (96, 16384, 256), (129, 200, 128),
                   (33, 6000, 256), (40, 16384, 128), (300, 4, 2432), (1000, 512, 64),
                   (8, 2048, 1024), (32, 300, 512), (64, 1002, 256), (40, 16388, 64), (64, 256, 100)]
 
 
+@pytest.mark.parametrize("wide", ["0", "1"])
 @pytest.mark.parametrize("mnk", REQUANT_SHAPES)
-def test_requantizing_linear_equals_linear_then_row_quantize(hip, mnk, knobs):
+def test_requantizing_linear_equals_linear_then_row_quantize(hip, mnk, wide, knobs):
     """vtl_hip_linear_i8_requant gives the codes, scales and (when asked for) f32 rows of
-    vtl_hip_linear_i8_f32 followed by the per-row quantizer, and of the oracle."""
+    vtl_hip_linear_i8_f32 followed by the per-row quantizer, and of the oracle.  `wide` picks
+    between the two forms of the launch without a K split (VTL_HIP_REQUANT_WIDE: row maxima in
+    the tile kernel's epilogue and a wide quantizer, or int32 sums and one workgroup per row)."""
+    knobs.setenv("VTL_HIP_REQUANT_WIDE", wide)
     m, n, k = mnk
     rng = np.random.Generator(np.random.Philox(m * 13 + n * 5 + k))
     a = rng.integers(-127, 128, (m, k), dtype=np.int8)

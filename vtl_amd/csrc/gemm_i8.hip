@@ -51,6 +51,10 @@ struct GemmArgs {
     // requant_scales, the f32 rows in `out` unless that is null.
     int8_t *requant_codes;
     float *requant_scales;
+    // Set by the launcher when the tile kernel itself applies the epilogue of a requantizing
+    // linear (no K split): [tiles along N][M] maxima of |y| over each tile's columns, which
+    // the tile kernel writes beside the f32 rows and requant_rows_wide_kernel reduces.
+    float *row_absmax_parts;
 };
 
 // LDS tiles are rows of BK bytes (BK/16 chunks of 16 bytes).  The chunk index
@@ -98,7 +102,7 @@ __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int bloc
 // over); every output element is
 //     y = fl(fl(f32(acc) * fl(sa*sw)) + bias), then ReLU,
 // evaluated in that order with separately rounded operations.
-template <int BM, int BN, int WM, int WN, bool F32OUT, bool EDGE, int NT>
+template <int BM, int BN, int WM, int WN, bool F32OUT, bool EDGE, int NT, bool ROWMAX = false>
 __device__ __forceinline__ void epilogue(v16i (&acc)[WM / 32][WN / 32], const GemmArgs &g, int m0, int n0,
                                          int wr, int wc, char *smem)
 {
@@ -137,6 +141,15 @@ __device__ __forceinline__ void epilogue(v16i (&acc)[WM / 32][WN / 32], const Ge
             s_bias[t] = g.bias ? g.bias[n] : 0.0f;
         }
         __syncthreads();
+        // ROWMAX: max |y| of every row of the wave tile over this lane's columns
+        float rmax[ROWMAX ? TM : 1][16];
+        if constexpr (ROWMAX) {
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    rmax[i][r] = 0.0f;
+        }
         // The bias / ReLU switches are uniform: branch once, not per element.
         auto store_tile = [&](auto has_bias_t, auto relu_t, auto nt_t) {
             constexpr bool HAS_BIAS = decltype(has_bias_t)::value;
@@ -165,6 +178,8 @@ __device__ __forceinline__ void epilogue(v16i (&acc)[WM / 32][WN / 32], const Ge
                                 y = y + bv;
                             if (RELU && y < 0.0f)
                                 y = 0.0f;
+                            if constexpr (ROWMAX)
+                                rmax[i][rq * 4 + k] = fmaxf(rmax[i][rq * 4 + k], fabsf(y));
                             float *dst = tile_out + ((unsigned)(ml + k) * (unsigned)N + (unsigned)nl);
                             if (NT_STORE)
                                 __builtin_nontemporal_store(y, dst);
@@ -198,7 +213,36 @@ __device__ __forceinline__ void epilogue(v16i (&acc)[WM / 32][WN / 32], const Ge
                     store_tile(F_{}, F_{}, nt_t);
             }
         };
-        if constexpr (BM == 256 && BN == 256) {
+        if constexpr (ROWMAX) {
+            store_all(F_{});   // the rows are read back by the next launch: cached stores
+            // Row maxima of the block tile: over the 32 lanes that hold a row's columns (DPP, the
+            // first five steps of wave_max: lanes 31 and 63 end up with their half's maximum),
+            // then over the waves side by side through LDS (behind the staged scales).
+            float *s_rm = s_bias + BN;   // [WN tiles along the row = BN / WN][BM]
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    float v = rmax[i][r];
+                    v = vtlhip::qdev::dpp_max_step<0xB1, 0xF>(v);
+                    v = vtlhip::qdev::dpp_max_step<0x4E, 0xF>(v);
+                    v = vtlhip::qdev::dpp_max_step<0x141, 0xF>(v);
+                    v = vtlhip::qdev::dpp_max_step<0x140, 0xF>(v);
+                    v = vtlhip::qdev::dpp_max_step<0x142, 0xA>(v);
+                    if ((lane & 31) == 31)
+                        s_rm[wc * BM + wr * WM + i * 32 + 8 * (r >> 2) + row_in + (r & 3)] = v;
+                }
+            __syncthreads();
+            const int tile_n = n0 / BN;
+            for (int t = threadIdx.x; t < BM; t += NT) {
+                float v = s_rm[t];
+#pragma unroll
+                for (int c = 1; c < BN / WN; c++)
+                    v = fmaxf(v, s_rm[c * BM + t]);
+                if (m0 + t < M)
+                    g.row_absmax_parts[(int64_t)tile_n * M + m0 + t] = v;
+            }
+        } else if constexpr (BM == 256 && BN == 256) {
             if (g.cached_out)
                 store_all(F_{});
             else
@@ -223,7 +267,7 @@ __device__ __attribute__((aligned(16))) int8_t g_zero_chunk[16];
 // Requires K % BK == 0, or with EDGE K % 16 == 0: then the chunks of the last
 // tile that lie past K are loaded as zeros, rows past M / N are clamped on load
 // and masked on store.
-template <int BM, int BN, int BK, int NSTAGE, int WR, int WC, bool F32OUT, bool EDGE, bool SPLIT>
+template <int BM, int BN, int BK, int NSTAGE, int WR, int WC, bool F32OUT, bool EDGE, bool SPLIT, bool ROWMAX = false>
 __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArgs g)
 {
     constexpr int NW = WR * WC, NT = 64 * NW;
@@ -481,7 +525,7 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArg
         gp.out = g.partials + (int64_t)split * M * N;
         epilogue<BM, BN, WM, WN, false, EDGE, NT>(acc, gp, m0, n0, wr, wc, smem);
     } else {
-        epilogue<BM, BN, WM, WN, F32OUT, EDGE, NT>(acc, g, m0, n0, wr, wc, smem);
+        epilogue<BM, BN, WM, WN, F32OUT, EDGE, NT, ROWMAX>(acc, g, m0, n0, wr, wc, smem);
     }
 }
 
@@ -554,14 +598,28 @@ __global__ __launch_bounds__(T) void finalize_requant_kernel(const GemmArgs g)
     __shared__ float red[NW];
     const int m = blockIdx.x, N = g.N;
     const int64_t mn = (int64_t)g.M * N;
+    // every load of the kernel is issued up front - the row scale, the column scales and bias
+    // of this thread's columns, then the int32 sums of all K ranges - so that the kernel is one
+    // memory latency deep, not three
     const float sa = g.sa[(int64_t)m * g.sa_stride];
-    // all loads of a K range are issued before the previous range is added: NV (x2) in flight
+    f4 swv[NV], bv[NV];
+#pragma unroll
+    for (int v = 0; v < NV; v++) {
+        const int n = 4 * (v * T + (int)threadIdx.x);
+        swv[v] = f4{0.f, 0.f, 0.f, 0.f};
+        bv[v] = f4{0.f, 0.f, 0.f, 0.f};
+        if (n < N) {
+            swv[v] = g.sw_stride ? *reinterpret_cast<const f4 *>(g.sw + n) : f4{g.sw[0], g.sw[0], g.sw[0], g.sw[0]};
+            if (g.bias)
+                bv[v] = *reinterpret_cast<const f4 *>(g.bias + n);
+        }
+    }
     v4i acc[NV];
     const int32_t *p0 = g.partials + (int64_t)m * N + 4 * (int)threadIdx.x;
 #pragma unroll
     for (int v = 0; v < NV; v++)
         acc[v] = 4 * (v * T + (int)threadIdx.x) < N ? *reinterpret_cast<const v4i *>(p0 + 4 * v * T) : v4i{0, 0, 0, 0};
-#pragma unroll 2
+#pragma unroll 4
     for (int s = 1; s < g.splits; s++) {
         v4i t[NV];
 #pragma unroll
@@ -579,14 +637,12 @@ __global__ __launch_bounds__(T) void finalize_requant_kernel(const GemmArgs g)
         const int n = 4 * (v * T + (int)threadIdx.x);
         y[v] = f4{0.f, 0.f, 0.f, 0.f};
         if (n < N) {
-            const f4 swv = g.sw_stride ? *reinterpret_cast<const f4 *>(g.sw + n) : f4{g.sw[0], g.sw[0], g.sw[0], g.sw[0]};
-            const f4 bv = g.bias ? *reinterpret_cast<const f4 *>(g.bias + n) : f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const float sc = sa * swv[j];
+                const float sc = sa * swv[v][j];
                 float t = (float)acc[v][j] * sc;
                 if (g.bias)
-                    t = t + bv[j];
+                    t = t + bv[v][j];
                 if (g.relu && t < 0.0f)
                     t = 0.0f;
                 y[v][j] = t;
@@ -638,6 +694,39 @@ int launch_finalize_requant(const GemmArgs &g, hipStream_t st)
     else
         hipLaunchKernelGGL((finalize_requant_kernel<1024, 4>), grid, dim3(1024), 0, st, g);
     return check_launch("finalize_requant_kernel");
+}
+
+// Second half of a requantizing linear whose tile kernel applied the epilogue itself: the
+// f32 rows are there, and per row one partial maximum of |y| per tile along N.  A workgroup
+// takes 4096 columns of one row: it reduces the row's partial maxima (a few hundred bytes,
+// every workgroup of the row redoes it), derives the row scale exactly as the row quantizer
+// does and writes the codes of its columns.  Needs N % 4 == 0 and 16-byte aligned rows.
+__global__ __launch_bounds__(256) void requant_rows_wide_kernel(const float *__restrict__ y,
+                                                                const float *__restrict__ parts, int tiles_n, int M,
+                                                                int N, int8_t *__restrict__ codes,
+                                                                float *__restrict__ scales)
+{
+    __shared__ float red[4];
+    const int m = blockIdx.y;
+    const int n = (int)blockIdx.x * 4096 + 4 * (int)threadIdx.x;
+    const f4 *row = reinterpret_cast<const f4 *>(y + (int64_t)m * N);
+    f4 v[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)   // in flight while the maxima are reduced
+        v[i] = n + 1024 * i < N ? row[(n + 1024 * i) >> 2] : f4{0.f, 0.f, 0.f, 0.f};
+    float am = 0.0f;
+    for (int t = threadIdx.x; t < tiles_n; t += 256)
+        am = fmaxf(am, parts[(int64_t)t * M + m]);
+    am = vtlhip::qdev::block_max<256>(am, red);
+    const float sy = am / 127.0f;
+    const vtlhip::qdev::QuantScale qp = vtlhip::qdev::make_quant_scale(sy);
+    if (blockIdx.x == 0 && threadIdx.x == 0)
+        scales[m] = sy;
+    unsigned *out = reinterpret_cast<unsigned *>(codes + (int64_t)m * N);
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+        if (n + 1024 * i < N)
+            out[(n + 1024 * i) >> 2] = vtlhip::qdev::quant4(v[i], qp);
 }
 
 // Weight-streaming kernel for M <= 32 (decode-shaped linear): bound by reading
@@ -1350,7 +1439,7 @@ template <int BM, int BN, int BK, int NSTAGE, int WR, int WC, bool F32OUT>
 int launch_dma(GemmArgs g, int splits, hipStream_t st)
 {
     constexpr int lds = NSTAGE * (BM + BN) * BK;
-    static_assert(lds >= (BM + 2 * BN) * 4, "epilogue staging fits in the operand buffers");
+    static_assert(lds >= (BM + 2 * BN + (BN / 32) * BM) * 4, "epilogue staging fits in the operand buffers");
     static_assert((NSTAGE - 1) * ((BM + BN) / (64 / (BK / 16)) / (WR * WC)) <= 63, "vmcnt is a 6-bit counter");
     const int tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
     const int kt_all = (g.K + BK - 1) / BK;
@@ -1366,14 +1455,53 @@ int launch_dma(GemmArgs g, int splits, hipStream_t st)
         if (!g.partials)
             return vtlhip::workspace_status();
     }
-    static PerDevice<bool> done_flags[6];
-    bool *done[6] = {&done_flags[0].get(), &done_flags[1].get(), &done_flags[2].get(),
-                     &done_flags[3].get(), &done_flags[4].get(), &done_flags[5].get()};
+    static PerDevice<bool> done_flags[8];
+    bool *done[8] = {&done_flags[0].get(), &done_flags[1].get(), &done_flags[2].get(), &done_flags[3].get(),
+                     &done_flags[4].get(), &done_flags[5].get(), &done_flags[6].get(), &done_flags[7].get()};
     const bool edge = (g.M % BM) || (g.N % BN) || (g.K % BK);
     g.cached_out = tiles <= 256 ? 1 : 0;  // one round of workgroups
     int rc;
     if (requant && splits == 1) {
-        // no K split: the int32 sums of the whole K go to the scratch plane the row kernel reads
+        // No K split.  Either the tile kernel applies the epilogue itself, leaves the f32 rows
+        // (in the caller's Y, or in the scratch plane) with one partial row maximum per tile, and
+        // a wide kernel quantizes them; or it leaves int32 sums and one workgroup per row does
+        // epilogue and quantization.  Measured, the second form is the faster one everywhere
+        // (256x11008x4096: 25.8 against 26.8 us, 128x14336x4096: 21.9 against 23.5 us,
+        // 256x16384x1024: 17.7 against 22.3 us; with the f32 rows wanted as well the gap is
+        // 0.6 to 1 us): the reduction in the tile kernel's epilogue and the second kernel's
+        // dependent loads cost more than the one-workgroup-per-row kernel's idle lanes.  So it
+        // is the default; VTL_HIP_REQUANT_WIDE=1 selects the first form (tests keep both exact).
+        constexpr bool kRowMaxTile = BM >= 64 && BM <= 128 && BN >= 64;   // the instantiated shapes
+        const int tiles_n = (g.N + BN - 1) / BN;
+        bool wide = kRowMaxTile && tuning().requant_wide > 0;
+        if constexpr (kRowMaxTile) {
+            if (wide) {
+                const size_t plane = (size_t)g.M * (size_t)g.N * sizeof(float);
+                char *ws = static_cast<char *>(
+                    vtlhip::library_workspace(plane + (size_t)tiles_n * (size_t)g.M * sizeof(float)));
+                if (!ws)
+                    return vtlhip::workspace_status();
+                GemmArgs gf = g;
+                gf.out = g.out ? g.out : reinterpret_cast<void *>(ws);
+                gf.row_absmax_parts = reinterpret_cast<float *>(ws + plane);
+                if (edge)
+                    rc = launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, true, true, false, true>,
+                                         *done[6], lds, tiles, 64 * WR * WC, gf, st, "gemm_i8_dma_kernel");
+                else
+                    rc = launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, true, false, false, true>,
+                                         *done[7], lds, tiles, 64 * WR * WC, gf, st, "gemm_i8_dma_kernel");
+                if (rc != VTL_HIP_OK)
+                    return rc;
+                const dim3 grid((unsigned)((g.N + 4095) / 4096), (unsigned)g.M);
+                if (grid.y > 65535)
+                    return VTL_HIP_ERR_UNSUPPORTED;
+                hipLaunchKernelGGL(requant_rows_wide_kernel, grid, dim3(256), 0, st,
+                                   reinterpret_cast<const float *>(gf.out), gf.row_absmax_parts, tiles_n, g.M, g.N,
+                                   g.requant_codes, g.requant_scales);
+                return check_launch("requant_rows_wide_kernel");
+            }
+        }
+        // the int32 sums of the whole K go to the scratch plane the row kernel reads
         GemmArgs gi = g;
         gi.out = g.partials;
         if (edge)

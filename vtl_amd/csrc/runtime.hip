@@ -68,6 +68,7 @@ static const Tuning *read_tuning(bool force)
         t->gemm_splits = splits;
     }
     t->no_fused_requant = flag("VTL_HIP_NO_FUSED_REQUANT");
+    t->requant_wide = number("VTL_HIP_REQUANT_WIDE", 0);
     t->no_fused_decode = flag("VTL_HIP_NO_FUSED_DECODE");
     t->skinny_tiled = number("VTL_HIP_SKINNY_TILED", -1);
     t->skinny_waves = number("VTL_HIP_SKINNY_WAVES", 4);
