@@ -1,0 +1,112 @@
+#!/usr/bin/env python3
+"""Writes tests/golden/gemm_tile_sweep.json: measured times of every tile configuration and
+K-split count of the int8 tile kernels for a handful of shapes, the ground truth that
+tests/test_gemm_tile_choice.py holds the library's cost model against.
+
+Run on the MI355X box from the repository root:
+
+    python3 tests/golden/make_gemm_tile_sweep.py > gpurun_out/gemm_tile_sweep.json
+
+and copy the result to tests/golden/gemm_tile_sweep.json.  Every (configuration, splits) pair
+is forced through VTL_HIP_GEMM_CONFIG and timed with HIP events over back-to-back launches,
+once re-reading the same weights (up to 256 MB of them stay in the last-level cache) and once
+taking the weights from enough copies in turn that every launch streams them from HBM.
+Shapes whose launch is a requantizing linear in the benchmark (the hidden layers of the MLP
+chain) are timed through vtl_hip_linear_i8_requant, the others through vtl_hip_linear_i8_f32.
+"""
+import ctypes as C
+import json
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, ROOT)
+from vtl_amd import capi  # noqa: E402
+from vtl_amd.tensor import HipTensor  # noqa: E402
+
+# (M, N, K, entry point): the tile-kernel launches of the five configurations, the two shapes an
+# earlier fit missed by 9-11 %, and a few in between
+SHAPES = [(4096, 4096, 4096, "linear"), (128, 14336, 4096, "linear"), (256, 11008, 4096, "requant"),
+          (256, 4096, 11008, "requant"), (6144, 6144, 2048, "linear"), (8192, 8192, 1024, "linear"),
+          (1024, 4096, 4096, "linear"), (64, 14336, 4096, "linear"), (2048, 2048, 2048, "linear"),
+          (512, 8192, 8192, "linear")]
+N_CONFIGS = 8
+SPLITS = (1, 2, 4, 8)
+
+
+def main():
+    capi.call("vtl_hip_set_device", 0)
+    e0, e1 = C.c_void_p(), C.c_void_p()
+    capi.call("vtl_hip_event_create", C.byref(e0))
+    capi.call("vtl_hip_event_create", C.byref(e1))
+    rng = np.random.Generator(np.random.Philox(11))
+    out = {"device": capi.device_info()[0], "unit": "us per launch", "shapes": []}
+    for m, n, k, entry in SHAPES:
+        w = rng.integers(-127, 128, (n, k), dtype=np.int8)
+        ncopy = max(2, min(16, -(-600_000_000 // (n * k))))
+        Ws = [HipTensor.from_host(w) for _ in range(ncopy)]
+        A = HipTensor.from_host(rng.integers(-127, 128, (m, k), dtype=np.int8))
+        sa = HipTensor.from_host(np.full(m, 0.01, np.float32))
+        sw = HipTensor.from_host(np.full(n, 0.01, np.float32))
+        Y = HipTensor.empty([m, n], np.float32)
+        Q = HipTensor.empty([m, n], np.int8)
+        S = HipTensor.empty([m], np.float32)
+        turn = [0]
+
+        def launch(streaming):
+            wt = Ws[turn[0] % ncopy] if streaming else Ws[0]
+            turn[0] += 1
+            if entry == "requant":
+                capi.call("vtl_hip_linear_i8_requant", A.ptr, sa.ptr, 1, wt.ptr, sw.ptr, 1, None, 1, Q.ptr, S.ptr,
+                          None, m, n, k)
+            else:
+                capi.call("vtl_hip_linear_i8_f32", A.ptr, sa.ptr, 1, wt.ptr, sw.ptr, 1, None, Y.ptr, m, n, k, 0)
+
+        def timed(streaming, reps):
+            best = 1e30
+            for _ in range(2):
+                for _ in range(10):
+                    launch(streaming)
+                capi.call("vtl_hip_sync")
+                capi.call("vtl_hip_event_record", e0)
+                for _ in range(reps):
+                    launch(streaming)
+                capi.call("vtl_hip_event_record", e1)
+                capi.call("vtl_hip_sync")
+                ms = C.c_float()
+                capi.call("vtl_hip_event_elapsed_ms", e0, e1, C.byref(ms))
+                best = min(best, ms.value / reps * 1e3)
+            return best
+
+        rec = {"m": m, "n": n, "k": k, "entry": entry, "weight_copies": ncopy, "cached": {}, "from_hbm": {}}
+        kt = (k + 127) // 128
+        for idx in range(N_CONFIGS):
+            for s in SPLITS:
+                if s > 1 and kt // s < 4:
+                    continue
+                os.environ["VTL_HIP_GEMM_CONFIG"] = f"{idx},{s}"
+                capi.call("vtl_hip_reload_env")
+                launch(False)
+                capi.call("vtl_hip_sync")
+                probe = timed(False, 5)
+                if probe > 2000.0:        # hopeless for this shape: not worth the minutes
+                    continue
+                reps = int(max(20, min(200, 4000.0 / probe)))
+                rec["cached"][f"{idx},{s}"] = round(timed(False, reps), 2)
+                rec["from_hbm"][f"{idx},{s}"] = round(timed(True, reps), 2)
+        os.environ.pop("VTL_HIP_GEMM_CONFIG", None)
+        capi.call("vtl_hip_reload_env")
+        rec["library_choice_cached"] = round(timed(False, 100), 2)
+        rec["library_choice_from_hbm"] = round(timed(True, 100), 2)
+        out["shapes"].append(rec)
+        print(f"{m}x{n}x{k} done", file=sys.stderr, flush=True)
+        for h in Ws + [A, sa, sw, Y, Q, S]:
+            h.release()
+    json.dump(out, sys.stdout, indent=1)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -47,3 +47,25 @@ def test_traffic_records_go_stale_with_their_source(tmp_path, monkeypatch):
     src.write_text("__global__ void k() { }\n")                 # the kernel changed after the counter run
     assert bench.measured_traffic("linear") is None
 
+
+
+def test_decode_and_chain_legs_time_the_configs_own_tensors():
+    """The timed tensors of configs[3] and configs[4] are the seeded ones of vtl_amd.workloads
+    (seeds 3 and 4), the same the parity tests and the golden fixtures use - no generator of
+    the benchmark's own."""
+    import importlib.util
+    import inspect
+    spec = importlib.util.spec_from_file_location("bench_under_test", os.path.join(ROOT, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    dec = inspect.getsource(bench._bench_decode)
+    chain = inspect.getsource(bench._bench_chain)
+    assert "workloads.decode_linear(" in dec and "workloads.decode_linear_activations(" in dec
+    assert "workloads.mlp_chain(" in chain
+    for src in (dec, chain, inspect.getsource(bench._other_decode_chain)):
+        assert "Philox" not in src and "default_rng" not in src and "rng." not in src
+    # and the activations bench.py draws for a given M are the ones decode_linear(M) returns
+    import numpy as np
+    from vtl_amd import workloads
+    x, _ = workloads.decode_linear(8, k=64, n=4)
+    assert np.array_equal(x, workloads.decode_linear_activations(8, k=64))

@@ -1984,6 +1984,11 @@ int vtl_hip_linear_i8_requant(const int8_t *A, const float *sa, int sa_per_row, 
         g.requant_scales = sy;
         int idx, splits;
         choose_config(M, N, K, idx, splits);
+        const Tuning &tn = tuning();
+        if (tn.gemm_config >= 0 && tn.gemm_config < kNumTileConfigs) {   // VTL_HIP_GEMM_CONFIG, as in launch_gemm
+            idx = tn.gemm_config;
+            splits = tn.gemm_splits;
+        }
         return launch_config<true>(idx, g, splits, current_stream());
     }
     // any other shape: the f32 rows (in the library's staging buffer when the caller wants none),
@@ -1998,6 +2003,21 @@ int vtl_hip_linear_i8_requant(const int8_t *A, const float *sa, int sa_per_row, 
     if (st != VTL_HIP_OK)
         return st;
     return launch_quantize_rows(Y, M, N, Yq, sy, current_stream());
+}
+
+int vtl_hip_gemm_tile_choice(int M, int N, int K, int *config_index, int *tile_m, int *tile_n, int *splits)
+{
+    if (!config_index || !tile_m || !tile_n || !splits || M <= 0 || N <= 0 || K <= 0)
+        return VTL_HIP_ERR_INVALID_ARG;
+    int idx, s;
+    choose_config(M, N, K, idx, s);
+    if (idx < 0)
+        return VTL_HIP_ERR_UNSUPPORTED;
+    *config_index = idx;
+    *tile_m = kTileConfigs[idx].bm;
+    *tile_n = kTileConfigs[idx].bn;
+    *splits = s;
+    return VTL_HIP_OK;
 }
 
 size_t vtl_hip_linear_f32_dynquant_workspace(int M, int K)
