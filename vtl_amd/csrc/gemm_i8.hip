@@ -10,6 +10,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 
+#include <atomic>
 #include <type_traits>
 
 #include "common.hpp"
@@ -1407,7 +1408,10 @@ __global__ __launch_bounds__(64 * NW) void gemm_i8_small_kernel(const GemmArgs g
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-// A value per device: kernel attributes are per device, the library may serve several.
+// A flag per device: kernel attributes are per device, the library may serve several.  Atomic,
+// so that two host threads that meet at a kernel's first launch do not race on the flag itself
+// (setting the attribute twice is harmless).
+using DoneFlag = std::atomic<bool>;
 template <typename V>
 struct PerDevice {
     V v[64] = {};
@@ -1423,13 +1427,13 @@ struct PerDevice {
 };
 
 template <typename Kern>
-int launch_with_lds(Kern kern, bool &attr_done, int lds, int tiles, int threads, const GemmArgs &g,
+int launch_with_lds(Kern kern, DoneFlag &attr_done, int lds, int tiles, int threads, const GemmArgs &g,
                     hipStream_t st, const char *name)
 {
-    if (!attr_done) {  // one host thread per device
+    if (!attr_done.load(std::memory_order_acquire)) {
         VTL_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-        attr_done = true;
+        attr_done.store(true, std::memory_order_release);
     }
     hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(threads), lds, st, g);
     return check_launch(name);
@@ -1455,8 +1459,8 @@ int launch_dma(GemmArgs g, int splits, hipStream_t st)
         if (!g.partials)
             return vtlhip::workspace_status();
     }
-    static PerDevice<bool> done_flags[8];
-    bool *done[8] = {&done_flags[0].get(), &done_flags[1].get(), &done_flags[2].get(), &done_flags[3].get(),
+    static PerDevice<DoneFlag> done_flags[8];
+    DoneFlag *done[8] = {&done_flags[0].get(), &done_flags[1].get(), &done_flags[2].get(), &done_flags[3].get(),
                      &done_flags[4].get(), &done_flags[5].get(), &done_flags[6].get(), &done_flags[7].get()};
     const bool edge = (g.M % BM) || (g.N % BN) || (g.K % BK);
     g.cached_out = tiles <= 256 ? 1 : 0;  // one round of workgroups
@@ -1642,15 +1646,15 @@ int launch_skinny_cfg(const GemmArgs &g, hipStream_t st)
 {
     constexpr int lds = NWAVE * STAGES * (8192 + XJ * 2048);
     static_assert(lds >= NWAVE * 4096, "room for the partial tiles");
-    static PerDevice<bool> done_flag;
-    bool &done = done_flag.get();
+    static PerDevice<DoneFlag> done_flag;
+    DoneFlag &done = done_flag.get();
     const dim3 grid((unsigned)((g.N + 31) / 32), (unsigned)((g.M + 31) / 32));
     if (grid.y > 65535)
         return VTL_HIP_ERR_UNSUPPORTED;
-    if (!done) {  // one host thread per device
+    if (!done.load(std::memory_order_acquire)) {
         VTL_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(linear_skinny_kernel<NWAVE, STAGES, XJ, F32OUT>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-        done = true;
+        done.store(true, std::memory_order_release);
     }
     hipLaunchKernelGGL((linear_skinny_kernel<NWAVE, STAGES, XJ, F32OUT>), grid, dim3(64 * NWAVE), lds, st, g);
     return check_launch("linear_skinny_kernel");

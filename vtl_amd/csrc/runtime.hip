@@ -93,7 +93,7 @@ const Tuning &tuning()
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 constexpr int kMaxDevices = 64;
-static void *g_scratch_ptr[kMaxDevices] = {};
+static std::atomic<void *> g_scratch_ptr[kMaxDevices] = {};
 
 static int current_device()
 {
@@ -110,16 +110,16 @@ void *static_scratch()
     const int dev = current_device();
     if (dev < 0)
         return nullptr;
-    if (!g_scratch_ptr[dev]) {
+    if (!g_scratch_ptr[dev].load(std::memory_order_acquire)) {   // two first callers resolve the same address
         void *ptr = nullptr;
         const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
         if (e != hipSuccess) {
             (void)record_hip_error(e, "hipGetSymbolAddress(scratch)");
             return nullptr;
         }
-        g_scratch_ptr[dev] = ptr;
+        g_scratch_ptr[dev].store(ptr, std::memory_order_release);
     }
-    return g_scratch_ptr[dev];
+    return g_scratch_ptr[dev].load(std::memory_order_acquire);
 }
 
 // While a ScratchArena is alive on this thread, library_workspace() hands out
