@@ -378,7 +378,13 @@ def bench_other_configs(timer: Timer, steps: int, warmup: int, cpu: bool = False
     configs[0] MNIST-MLP first layer, configs[3] decode-shaped linear with
     per-token quantization on the fly, configs[4] 3-layer int8 MLP chain."""
     from vtl_amd.storage import HipStorage
-    out = {}
+    # These are side figures, not `value`: launches of 4 to 60 us whose first few dozen after an idle
+    # spell run 5-15 % slow while the card's clocks settle, so they are timed over at least 100
+    # launches after at least 100 warm-up launches whatever --steps / --warmup say (the headline
+    # and the quantize / dequantize legs use --steps / --warmup exactly).
+    warmup, steps = max(warmup, 100), max(steps, 100)
+    out = {"note": f"every figure in here: {steps} timed launches after {warmup} warm-up launches "
+                   "(at least 100 of each; see bench.py)"}
 
     def timed(fn):
         for _ in range(warmup):
