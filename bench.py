@@ -373,7 +373,7 @@ def bench_quant(timer: Timer, steps: int, warmup: int, cpu: bool):
 
 
 def bench_other_configs(timer: Timer, steps: int, warmup: int, cpu: bool = False, parts=("mnist", "decode", "chain"),
-                        decode_cached: bool = True):
+                        decode_cached: bool = True, exact: bool = False):
     """Timings of the remaining configurations (parity for them is in tests/):
     configs[0] MNIST-MLP first layer, configs[3] decode-shaped linear with
     per-token quantization on the fly, configs[4] 3-layer int8 MLP chain."""
@@ -382,9 +382,10 @@ def bench_other_configs(timer: Timer, steps: int, warmup: int, cpu: bool = False
     # spell run 5-15 % slow while the card's clocks settle, so they are timed over at least 100
     # launches after at least 100 warm-up launches whatever --steps / --warmup say (the headline
     # and the quantize / dequantize legs use --steps / --warmup exactly).
-    warmup, steps = max(warmup, 100), max(steps, 100)
+    if not exact:
+        warmup, steps = max(warmup, 100), max(steps, 100)
     out = {"note": f"every figure in here: {steps} timed launches after {warmup} warm-up launches "
-                   "(at least 100 of each; see bench.py)"}
+                   "(at least 100 of each unless --other-exact; see bench.py)"}
 
     def timed(fn):
         for _ in range(warmup):
@@ -752,6 +753,8 @@ def main() -> int:
     ap.add_argument("--vendor-yardstick-child", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--no-vendor-yardstick", action="store_true",
                     help="skip the torch._int_mm timing printed beside the Linear")
+    ap.add_argument("--other-exact", action="store_true",
+                    help="time the side figures over exactly --steps / --warmup launches (short profiling runs)")
     ap.add_argument("--decode-from-hbm-only", action="store_true",
                     help="with --only decode: skip the launches that re-read the same weights (profiling)")
     args = ap.parse_args()
@@ -775,11 +778,12 @@ def main() -> int:
         print(json.dumps({"full_precision": bench_full_precision(timer, args.steps, args.warmup)}))
         return 0
     if args.only == "other":
-        print(json.dumps({"other_configs": bench_other_configs(timer, args.steps, args.warmup, cpu)}))
+        print(json.dumps({"other_configs": bench_other_configs(timer, args.steps, args.warmup, cpu,
+                                                               exact=args.other_exact)}))
         return 0
     if args.only in ("decode", "chain"):
         print(json.dumps({"other_configs": bench_other_configs(timer, args.steps, args.warmup, False, (args.only,),
-                                                               not args.decode_from_hbm_only)}))
+                                                               not args.decode_from_hbm_only, args.other_exact)}))
         return 0
     if args.only == "mfma":
         print(json.dumps({"mfma_only": bench_mfma_only(timer, max(args.load_seconds, 0.05))}))
@@ -830,7 +834,7 @@ def main() -> int:
         if not args.no_vendor_yardstick:
             line["vendor_int8_mm"] = bench_vendor_yardstick(args.steps, args.warmup)
     if args.only == "all":
-        line["other_configs"] = bench_other_configs(timer, args.steps, args.warmup, cpu)
+        line["other_configs"] = bench_other_configs(timer, args.steps, args.warmup, cpu, exact=args.other_exact)
         line["full_precision"] = bench_full_precision(timer, args.steps, args.warmup)
     print(json.dumps(line))
     return 0
