@@ -223,3 +223,71 @@ def test_v_binding_declarations_match_the_header():
                  "vtl_hip_linear_i8_requant", "vtl_hip_linear_f32_dynquant", "vtl_hip_matmul_f32", "vtl_hip_linear_backward_f32",
                  "vtl_hip_malloc", "vtl_hip_free", "vtl_hip_memcpy_h2d", "vtl_hip_memcpy_d2h"):
         assert must in seen, must
+
+
+def _v_files():
+    vbind = os.path.join(ROOT, "vtl_amd", "vbind")
+    for dirpath, _, files in os.walk(vbind):
+        for f in sorted(files):
+            if f.endswith(".v"):
+                yield os.path.join(dirpath, f)
+
+
+def _strip_v_comments_and_strings(text):
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"//[^\n]*", "", text)
+    text = re.sub(r"'(?:\\.|[^'\\\n])*'", "''", text)
+    text = re.sub(r'"(?:\\.|[^"\\\n])*"', '""', text)
+    return re.sub(r"`(?:\\.|[^`\\\n])`", "``", text)
+
+
+def _pub_fns(text):
+    """name (with receiver type) -> normalised parameter list and return type of every `pub fn`."""
+    out = {}
+    code = _strip_v_comments_and_strings(text)
+    for recv, name, params, ret in re.findall(
+            r"^pub fn\s*(\([^)]*\)\s*)?(\w+)(?:\[[^\]]*\])?\(([^)]*)\)\s*([^{\n]*)\{", code, flags=re.M):
+        recv_type = re.sub(r"^\(\s*(?:mut\s+)?\w+\s+", "", recv.strip()).rstrip(") ").strip() if recv else ""
+        types = [re.sub(r"^(?:mut\s+)?\w+\s+", "", p.strip()) for p in params.split(",") if p.strip()]
+        out[(recv_type, name)] = (tuple(types), ret.strip())
+    return out
+
+
+def test_v_binding_files_are_balanced_and_flag_pairs_define_the_same_public_functions():
+    """No V compiler exists in this image, so the binding files get the checks that need none:
+    every file starts with its module line and has balanced brackets outside comments and
+    strings, and a `_d_hip.v` / `_notd_hip.v` pair - of which the V build compiles exactly one,
+    depending on `-d hip` - defines the same public functions with the same parameter and
+    return types (cf. storage/cuda_d_cuda.v against storage/cuda_notd_cuda.v)."""
+    files = list(_v_files())
+    assert len(files) >= 20
+    for path in files:
+        text = open(path).read()
+        first = [l for l in text.splitlines() if l.strip() and not l.strip().startswith("//")][0]
+        assert first.startswith("module "), path
+        code = _strip_v_comments_and_strings(text)
+        for a, b in ("()", "{}", "[]"):
+            assert code.count(a) == code.count(b), f"{path}: unbalanced {a}{b}"
+    pairs = 0
+    for path in files:
+        if not path.endswith("_d_hip.v"):
+            continue
+        twin = path[:-len("_d_hip.v")] + "_notd_hip.v"
+        if not os.path.exists(twin):
+            continue
+        pairs += 1
+        d, n = _pub_fns(open(path).read()), _pub_fns(open(twin).read())
+        # the stub side may be a subset only where the `-d hip` side adds device-only helpers that
+        # nothing outside `$if hip ? {}` calls; what both define must agree exactly
+        # (the device tensor type exists only with `-d hip`: where the real function returns
+        # &HipTensor[T] / &HipStorage[T] the stub returns &Tensor[T] / &CpuStorage[T], as
+        # tensor_cuda_notd_cuda.v:12-15 and storage/cuda_notd_cuda.v:13-16 do)
+        def device_to_host(t):
+            return t.replace("HipTensor[", "Tensor[").replace("HipStorage[", "CpuStorage[")
+        norm = lambda sig: (tuple(device_to_host(t) for t in sig[0]), device_to_host(sig[1]))   # noqa: E731
+        for key in sorted(set(d) & set(n)):
+            assert norm(d[key]) == norm(n[key]), \
+                f"{os.path.basename(path)}: {key[1]} differs from its stub: {d[key]} vs {n[key]}"
+        missing = sorted(k[1] for k in set(n) - set(d))
+        assert not missing, f"{os.path.basename(twin)} defines {missing}, its `-d hip` twin does not"
+    assert pairs >= 6
