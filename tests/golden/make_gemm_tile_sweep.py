@@ -5,9 +5,9 @@ tests/test_gemm_tile_choice.py holds the library's cost model against.
 
 Run on the MI355X box from the repository root:
 
-    python3 tests/golden/make_gemm_tile_sweep.py > gpurun_out/gemm_tile_sweep.json
+    python3 tests/golden/make_gemm_tile_sweep.py > gemm_tile_sweep.json
 
-and copy the result to tests/golden/gemm_tile_sweep.json.  Every (configuration, splits) pair
+and put the result at tests/golden/gemm_tile_sweep.json.  Every (configuration, splits) pair
 is forced through VTL_HIP_GEMM_CONFIG and timed with HIP events over back-to-back launches,
 once re-reading the same weights (up to 256 MB of them stay in the last-level cache) and once
 taking the weights from enough copies in turn that every launch streams them from HBM.
