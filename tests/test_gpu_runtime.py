@@ -183,6 +183,69 @@ def test_entry_points_capture_into_a_hip_graph(hip):
             t.release()
 
 
+def test_library_scratch_recorded_into_a_graph_survives_growth_and_never_grows_under_capture(hip):
+    """vtl_hip_linear_f32_dynquant without a caller workspace stages the activation codes in the
+    library's own buffer, whose address a stream capture bakes into the graph.  A later eager
+    call that needs a larger buffer must not free the recorded one (replays still write to it),
+    and a call that would have to grow the buffer during a capture is refused with a status."""
+    import oracle
+    hiprt = C.CDLL("libamdhip64.so")
+    stream, graph, gexec = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    assert hiprt.hipStreamCreate(C.byref(stream)) == 0
+    rng = np.random.default_rng(63)
+    m, n, k = 40, 256, 1024
+    w = rng.integers(-127, 128, (n, k), dtype=np.int8)
+    sw = rng.uniform(0.5, 1.5, n).astype(np.float32)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    X, W, SW = (HipTensor.from_host(a) for a in (x, w, sw))
+    Y = HipTensor.empty([m, n], np.float32)
+    # the eager call that makes the staging buffer grow: 96 MiB of codes, more than any other test stages
+    mb, kb = 24576, 4096
+    XB = HipTensor.empty([mb, kb], np.float32)
+    WB = HipTensor.from_host(rng.integers(-127, 128, (64, kb), dtype=np.int8))
+    YB = HipTensor.empty([mb, 64], np.float32)
+    capi.call("vtl_hip_memset", XB.ptr, 0, mb * kb * 4)
+    mc = 40960                                      # 160 MiB of codes: asked for under capture only
+    XC, YC = HipTensor.empty([mc, kb], np.float32), HipTensor.empty([mc, 64], np.float32)
+
+    def small():
+        capi.call("vtl_hip_linear_f32_dynquant", X.ptr, W.ptr, SW.ptr, None, Y.ptr, m, n, k, 0, None, 0)
+
+    try:
+        capi.call("vtl_hip_set_stream", stream)
+        small()                                     # warm-up: the buffer exists, kernel attributes are set
+        capi.call("vtl_hip_sync")
+        assert hiprt.hipStreamBeginCapture(stream, 0) == 0
+        small()
+        assert hiprt.hipStreamEndCapture(stream, C.byref(graph)) == 0
+        assert hiprt.hipGraphInstantiate(C.byref(gexec), graph, None, None, C.c_size_t(0)) == 0
+        capi.call("vtl_hip_linear_f32_dynquant", XB.ptr, WB.ptr, SW.ptr, None, YB.ptr, mb, 64, kb, 0, None, 0)
+        capi.call("vtl_hip_sync")
+        for rep in range(3):
+            xr = (rng.standard_normal((m, k)) * (rep + 2)).astype(np.float32)
+            capi.call("vtl_hip_memcpy_h2d", X.ptr, xr.ctypes.data, xr.nbytes)
+            assert hiprt.hipGraphLaunch(gexec, stream) == 0
+            capi.call("vtl_hip_sync")
+            assert np.array_equal(Y.cpu(), oracle.linear_f32_dynquant(xr, w, sw, None)), f"replay {rep}"
+        # under capture the buffer may be used, never grown: 160 MiB of codes do not fit what exists
+        assert hiprt.hipStreamBeginCapture(stream, 0) == 0
+        st = capi.status("vtl_hip_linear_f32_dynquant", XC.ptr, WB.ptr, SW.ptr, None, YC.ptr, mc, 64, kb, 0, None, 0)
+        graph2 = C.c_void_p()
+        assert hiprt.hipStreamEndCapture(stream, C.byref(graph2)) == 0
+        if graph2:
+            hiprt.hipGraphDestroy(graph2)
+        assert st == capi.ERR_UNSUPPORTED and b"stream capture" in capi.lib().vtl_hip_last_error()
+    finally:
+        capi.call("vtl_hip_set_stream", None)
+        if gexec:
+            hiprt.hipGraphExecDestroy(gexec)
+        if graph:
+            hiprt.hipGraphDestroy(graph)
+        hiprt.hipStreamDestroy(stream)
+        for t in (X, W, SW, Y, XB, WB, YB, XC, YC):
+            t.release()
+
+
 def test_mfma_probe_runs_and_leaves_its_sink_alone(hip):
     """The measurement aid behind bench.py's `mfma_only` figures: launches, finishes, and
     never writes its sink (the sums it keeps alive cannot reach the sentinel)."""
