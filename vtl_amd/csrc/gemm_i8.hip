@@ -103,9 +103,40 @@ __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int bloc
 // over); every output element is
 //     y = fl(fl(f32(acc) * fl(sa*sw)) + bias), then ReLU,
 // evaluated in that order with separately rounded operations.
+// Scales and bias of a block tile, fetched by the threads of the workgroup before the K loop
+// (thread t takes rows / columns t, t + NT, ...) and put into LDS by the epilogue: read only
+// then, they add a memory latency to the end of every workgroup.  Used by the 256x256 tile
+// (4096^3: 0.3 to 1 us earlier); the smaller tiles measured no better with it and read them
+// in the epilogue.
+template <int BM>
+constexpr bool kScalesAhead = BM == 256;
+
+template <int BM, int BN, int NT>
+struct EpilogueScales {
+    float sa[(BM + NT - 1) / NT], sw[(BN + NT - 1) / NT], bias[(BN + NT - 1) / NT];
+};
+
+template <int BM, int BN, int NT, bool EDGE>
+__device__ __forceinline__ void fetch_scales(EpilogueScales<BM, BN, NT> &e, const GemmArgs &g, int m0, int n0)
+{
+#pragma unroll
+    for (int i = 0; i < (BM + NT - 1) / NT; i++) {
+        const int t = (int)threadIdx.x + i * NT;
+        const int m = EDGE ? min(m0 + t, g.M - 1) : m0 + t;
+        e.sa[i] = t < BM ? g.sa[(int64_t)m * g.sa_stride] : 0.0f;
+    }
+#pragma unroll
+    for (int i = 0; i < (BN + NT - 1) / NT; i++) {
+        const int t = (int)threadIdx.x + i * NT;
+        const int n = EDGE ? min(n0 + t, g.N - 1) : n0 + t;
+        e.sw[i] = t < BN ? g.sw[(int64_t)n * g.sw_stride] : 0.0f;
+        e.bias[i] = (t < BN && g.bias) ? g.bias[n] : 0.0f;
+    }
+}
+
 template <int BM, int BN, int WM, int WN, bool F32OUT, bool EDGE, int NT, bool ROWMAX = false>
 __device__ __forceinline__ void epilogue(v16i (&acc)[WM / 32][WN / 32], const GemmArgs &g, int m0, int n0,
-                                         int wr, int wc, char *smem)
+                                         int wr, int wc, char *smem, const EpilogueScales<BM, BN, NT> &pre)
 {
     constexpr int TM = WM / 32, TN = WN / 32;
     const int lane = threadIdx.x & 63;
@@ -132,14 +163,27 @@ __device__ __forceinline__ void epilogue(v16i (&acc)[WM / 32][WN / 32], const Ge
         float *s_sw = s_sa + BM;                        // [BN]
         float *s_bias = s_sw + BN;                      // [BN]
         __syncthreads();  // every wave is done with the operand tiles
-        for (int t = threadIdx.x; t < BM; t += NT) {
-            const int m = EDGE ? min(m0 + t, M - 1) : m0 + t;
-            s_sa[t] = g.sa[(int64_t)m * g.sa_stride];
-        }
-        for (int t = threadIdx.x; t < BN; t += NT) {
-            const int n = EDGE ? min(n0 + t, N - 1) : n0 + t;
-            s_sw[t] = g.sw[(int64_t)n * g.sw_stride];
-            s_bias[t] = g.bias ? g.bias[n] : 0.0f;
+        if constexpr (kScalesAhead<BM>) {
+#pragma unroll
+            for (int i = 0; i < (BM + NT - 1) / NT; i++)
+                if ((int)threadIdx.x + i * NT < BM)
+                    s_sa[threadIdx.x + i * NT] = pre.sa[i];
+#pragma unroll
+            for (int i = 0; i < (BN + NT - 1) / NT; i++)
+                if ((int)threadIdx.x + i * NT < BN) {
+                    s_sw[threadIdx.x + i * NT] = pre.sw[i];
+                    s_bias[threadIdx.x + i * NT] = pre.bias[i];
+                }
+        } else {
+            for (int t = threadIdx.x; t < BM; t += NT) {
+                const int m = EDGE ? min(m0 + t, M - 1) : m0 + t;
+                s_sa[t] = g.sa[(int64_t)m * g.sa_stride];
+            }
+            for (int t = threadIdx.x; t < BN; t += NT) {
+                const int n = EDGE ? min(n0 + t, N - 1) : n0 + t;
+                s_sw[t] = g.sw[(int64_t)n * g.sw_stride];
+                s_bias[t] = g.bias ? g.bias[n] : 0.0f;
+            }
         }
         __syncthreads();
         // ROWMAX: max |y| of every row of the wave tile over this lane's columns
@@ -343,6 +387,10 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArg
                                              0, 0);
     };
 
+    EpilogueScales<BM, BN, NT> pre;
+    if constexpr (F32OUT && !SPLIT && kScalesAhead<BM>)
+        fetch_scales<BM, BN, NT, EDGE>(pre, g, m0, n0);
+
     v16i acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; i++)
@@ -524,9 +572,9 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArg
         // raw partial sums of this K range; splitk_finalize_kernel adds the ranges up
         GemmArgs gp = g;
         gp.out = g.partials + (int64_t)split * M * N;
-        epilogue<BM, BN, WM, WN, false, EDGE, NT>(acc, gp, m0, n0, wr, wc, smem);
+        epilogue<BM, BN, WM, WN, false, EDGE, NT>(acc, gp, m0, n0, wr, wc, smem, pre);
     } else {
-        epilogue<BM, BN, WM, WN, F32OUT, EDGE, NT, ROWMAX>(acc, g, m0, n0, wr, wc, smem);
+        epilogue<BM, BN, WM, WN, F32OUT, EDGE, NT, ROWMAX>(acc, g, m0, n0, wr, wc, smem, pre);
     }
 }
 
@@ -817,6 +865,25 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_skinny_kernel(const GemmArg
         xoff[s] = xrow * BK + ((((2 * s + fh) ^ xrow) & 15) << 4);
     }
 
+    // The scales and bias of the outputs this thread will write are asked for now, ahead of the
+    // weight stream: read in the epilogue they would add a memory latency to the end of every
+    // workgroup.  (They are older than every ring load, so the ring's vmcnt waits cover them.)
+    constexpr int ITEMS = 256 / (64 * NWAVE);   // (m, 4 x n) outputs per thread
+    float e_sa[F32OUT ? ITEMS : 1], e_sw[F32OUT ? ITEMS : 1][4], e_bias[F32OUT ? ITEMS : 1][4];
+    if constexpr (F32OUT) {
+#pragma unroll
+        for (int it = 0; it < ITEMS; it++) {
+            const int item = tid + it * 64 * NWAVE;
+            const int m = m0 + (item >> 3), n = n0 + (item & 7) * 4;
+            e_sa[it] = m < M ? g.sa[(int64_t)m * g.sa_stride] : 0.0f;
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const bool in = m < M && n + k < N;
+                e_sw[it][k] = in ? g.sw[(int64_t)(n + k) * g.sw_stride] : 0.0f;
+                e_bias[it][k] = (in && g.bias) ? g.bias[n + k] : 0.0f;
+            }
+        }
+    }
 #pragma unroll
     for (int st = 0; st < STAGES - 1; st++)
         if (st < KC)
@@ -864,7 +931,9 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_skinny_kernel(const GemmArg
     }
     __syncthreads();
     // 256 (m, 4 x n) items; 8 threads cover the 128-byte row segment of one m
-    for (int item = tid; item < 256; item += 64 * NWAVE) {
+#pragma unroll
+    for (int it = 0; it < ITEMS; it++) {
+        const int item = tid + it * 64 * NWAVE;
         const int ml = item >> 3, nq = (item & 7) * 4;
         v4i sum = *reinterpret_cast<const v4i *>(part + ml * 32 + nq);
 #pragma unroll
@@ -876,15 +945,15 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_skinny_kernel(const GemmArg
         const int n = n0 + nq;
         const int64_t o = (int64_t)m * N + n;
         if constexpr (F32OUT) {
-            const float a = g.sa[(int64_t)m * g.sa_stride];
+            const float a = e_sa[it];
             float y[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int k = 0; k < 4; k++) {
                 if (n + k < N) {
-                    const float sc = a * g.sw[(int64_t)(n + k) * g.sw_stride];
+                    const float sc = a * e_sw[it][k];
                     float v = (float)sum[k] * sc;
                     if (g.bias)
-                        v = v + g.bias[n + k];
+                        v = v + e_bias[it][k];
                     if (g.relu && v < 0.0f)
                         v = 0.0f;
                     y[k] = v;
