@@ -163,7 +163,13 @@ int vtl_hip_linear_i8_requant(const int8_t *A, const float *sa, int sa_per_row,
  * aligned, owned by the caller (the reference's DeviceSession keeps such
  * staging buffers, autograd_cuda/device_session.v:13-24); NULL (with size 0)
  * makes the library stage in a buffer of its own, one per device, grown on
- * demand. */
+ * demand.  Calls that may overlap on a device (several streams) need a
+ * workspace each.  For 2 to 32 rows against at least 2048 weight rows
+ * (K % 256 == 0, K <= 8192) quantizer and linear are one launch whose
+ * workgroups meet on a device counter that the library keeps per stream, for
+ * the first 16 streams that make such a call; calls on further streams, and
+ * calls made while the stream is being captured into a graph, are two
+ * launches with the same results. */
 size_t vtl_hip_linear_f32_dynquant_workspace(int M, int K);
 int vtl_hip_linear_f32_dynquant(const float *X, const int8_t *Wq, const float *sw,
                                 const float *bias, float *Y, int M, int N, int K, int relu,

@@ -1,5 +1,7 @@
 """GPU parity of the layer-level path (linear_forward_f32 hook, QuantLinearLayer,
 Sequential) on the benchmark configurations, through the host-side mirror."""
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -270,6 +272,138 @@ def test_few_token_fused_decode_equals_two_launch_path(hip, mnk, knobs):
         S.release()
     for h in (X, W, SW, B):
         h.release()
+
+
+@pytest.mark.parametrize("mnk", [(2, 2048, 256), (8, 14336, 4096), (8, 2077, 1280), (9, 3001, 512), (16, 2048, 8192),
+                                 (17, 4096, 2048), (31, 2050, 4096), (32, 14336, 4096)])
+def test_decode_launch_that_quantizes_its_rows_equals_two_launch_path(hip, mnk, knobs):
+    """2 to 32 tokens against thousands of weight rows: one launch whose first workgroups
+    quantize the rows while the others wait for them.  Same bits as quantizer + linear and as
+    the oracle, special values included; also when no workgroup waits at all (spin limit 0:
+    every workgroup quantizes the rows itself) or waits for one poll only, and when the same
+    staging buffer is used again for other activations."""
+    m, n, k = mnk
+    rng = np.random.Generator(np.random.Philox(m * 11 + n + k))
+    w = rng.integers(-127, 128, (n, k), dtype=np.int8)
+    sw = (rng.uniform(0.5, 1.5, n) * 1e-3).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    W, SW, B = dev(w), dev(sw), dev(bias)
+    session = HipSession()
+    need = int(capi.lib().vtl_hip_linear_f32_dynquant_workspace(m, k))
+    ws = session.ensure("dynquant", need)
+    xs = []
+    for variant in range(3):
+        x = (rng.standard_normal((m, k), dtype=np.float32) * np.float32(variant + 1))
+        x[0, :4] = [0.5, 1.5, -2.5, 3.5]
+        x[m - 1] *= np.float32(1e-30)            # a row with a tiny scale
+        if variant == 1:
+            x[m // 2] = 0.0                      # an all-zero row: scale 0, codes 0
+        xs.append(x)
+    for special in (np.nan, np.inf, -np.inf):
+        x = xs[0].copy()
+        x[0, 7] = special
+        x[m - 1, k - 1] = special
+        xs.append(x)
+    wants = [oracle.linear_f32_dynquant(x, w, sw, bias, relu=True, threads=CPU_THREADS) for x in xs]
+    for spin in (None, "0", "1", "two launches"):
+        if spin == "two launches":
+            knobs.setenv("VTL_HIP_NO_FUSED_DECODE", "1")
+        elif spin is not None:
+            knobs.setenv("VTL_HIP_STAGE_SPIN", spin)
+        for x, want in zip(xs, wants):           # the same staging buffer, other activations
+            X = dev(x)
+            got = linear_f32_dynquant_hip(X, W, SW, B, relu=True, workspace=ws).cpu()
+            assert np.array_equal(got, want, equal_nan=True), (spin, mnk)
+            X.release()
+        knobs.delenv("VTL_HIP_STAGE_SPIN", raising=False)
+        knobs.delenv("VTL_HIP_NO_FUSED_DECODE", raising=False)
+    session.release()
+    for h in (W, SW, B):
+        h.release()
+
+
+def test_decode_launch_counters_are_per_stream_and_run_out_gracefully(hip):
+    """The workgroups of that launch meet on a counter the library keeps per stream (16 of
+    them): calls that alternate between streams, and calls on more streams than there are
+    counters (those take the two-launch path), all give the oracle's bits."""
+    hiprt = C.CDLL("libamdhip64.so")
+    m, n, k = 8, 2048, 512
+    rng = np.random.Generator(np.random.Philox(77))
+    w = rng.integers(-127, 128, (n, k), dtype=np.int8)
+    sw = (rng.uniform(0.5, 1.5, n) * 1e-3).astype(np.float32)
+    W, SW = dev(w), dev(sw)
+    streams = []
+    try:
+        for i in range(20):
+            st = C.c_void_p()
+            assert hiprt.hipStreamCreate(C.byref(st)) == 0
+            streams.append(st)
+        for rnd in range(3):
+            for i, st in enumerate(streams):
+                x = rng.standard_normal((m, k), dtype=np.float32) * np.float32(i + 1)
+                X = dev(x)
+                Y = HipTensor.empty([m, n], np.float32)
+                capi.call("vtl_hip_set_stream", st)
+                capi.call("vtl_hip_linear_f32_dynquant", X.ptr, W.ptr, SW.ptr, None, Y.ptr, m, n, k, 0, None, 0)
+                capi.call("vtl_hip_sync")
+                assert np.array_equal(Y.cpu(), oracle.linear_f32_dynquant(x, w, sw, None)), (rnd, i)
+                X.release()
+                Y.release()
+    finally:
+        capi.call("vtl_hip_set_stream", None)
+        for st in streams:
+            hiprt.hipStreamDestroy(st)
+        W.release()
+        SW.release()
+
+
+def test_decode_launch_is_replaced_by_two_launches_under_stream_capture(hip):
+    """A graph replays the kernel arguments it recorded, and the launch that quantizes its own
+    rows waits for a counter value that is new on every call: under capture the library records
+    quantizer + linear instead, and every replay gives the oracle's bits."""
+    hiprt = C.CDLL("libamdhip64.so")
+    stream, graph, gexec = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    assert hiprt.hipStreamCreate(C.byref(stream)) == 0
+    m, n, k = 16, 4096, 1024
+    rng = np.random.Generator(np.random.Philox(78))
+    w = rng.integers(-127, 128, (n, k), dtype=np.int8)
+    sw = (rng.uniform(0.5, 1.5, n) * 1e-3).astype(np.float32)
+    x = rng.standard_normal((m, k), dtype=np.float32)
+    X, W, SW = dev(x), dev(w), dev(sw)
+    Y = HipTensor.empty([m, n], np.float32)
+
+    def call():
+        capi.call("vtl_hip_linear_f32_dynquant", X.ptr, W.ptr, SW.ptr, None, Y.ptr, m, n, k, 0, None, 0)
+
+    try:
+        capi.call("vtl_hip_set_stream", stream)
+        call()                                      # eager: the one-launch form; the staging buffer exists now
+        capi.call("vtl_hip_sync")
+        assert np.array_equal(Y.cpu(), oracle.linear_f32_dynquant(x, w, sw, None))
+        assert hiprt.hipStreamBeginCapture(stream, 0) == 0
+        call()
+        assert hiprt.hipStreamEndCapture(stream, C.byref(graph)) == 0
+        assert hiprt.hipGraphInstantiate(C.byref(gexec), graph, None, None, C.c_size_t(0)) == 0
+        for rep in range(4):
+            xr = (rng.standard_normal((m, k)) * (rep + 2)).astype(np.float32)
+            capi.call("vtl_hip_memcpy_h2d", X.ptr, xr.ctypes.data, xr.nbytes)
+            if rep % 2:
+                call()                              # eager calls between the replays, on the same stream
+                capi.call("vtl_hip_sync")
+                assert np.array_equal(Y.cpu(), oracle.linear_f32_dynquant(xr, w, sw, None)), f"eager {rep}"
+                capi.call("vtl_hip_memset", Y.ptr, 0, m * n * 4)
+            assert hiprt.hipGraphLaunch(gexec, stream) == 0
+            capi.call("vtl_hip_sync")
+            assert np.array_equal(Y.cpu(), oracle.linear_f32_dynquant(xr, w, sw, None)), f"replay {rep}"
+    finally:
+        capi.call("vtl_hip_set_stream", None)
+        if gexec:
+            hiprt.hipGraphExecDestroy(gexec)
+        if graph:
+            hiprt.hipGraphDestroy(graph)
+        hiprt.hipStreamDestroy(stream)
+        for t in (X, W, SW, Y):
+            t.release()
 
 
 @pytest.mark.parametrize("nk", [(2048, 256), (2050, 512), (3001, 4096), (2077, 1280), (1, 16), (7, 48), (300, 784),

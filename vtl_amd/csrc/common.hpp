@@ -64,6 +64,7 @@ struct Tuning {
     bool no_fused_requant = false;  // VTL_HIP_NO_FUSED_REQUANT: linear, then the row quantizer
     int requant_wide = 0;           // VTL_HIP_REQUANT_WIDE: 1 row maxima in the tile kernel + wide quantizer, 0 one workgroup per row
     bool no_fused_decode = false;   // VTL_HIP_NO_FUSED_DECODE: quantizer launch in front of the linear
+    int stage_spin = 4096;          // VTL_HIP_STAGE_SPIN: polls a workgroup of the decode launch waits for the quantized rows (0: none, tests)
     int skinny_tiled = -1;          // VTL_HIP_SKINNY_TILED: 1 / 0 force the 32x32-block weight-streaming kernel for M > 32
     int skinny_waves = 4;           // VTL_HIP_SKINNY_WAVES: 2, 4 or 8 waves (K ranges) per workgroup there
     int matmul_tile = 0;            // VTL_HIP_MATMUL_TILE: 128 / 64 force the f64-accumulating tile

@@ -11,6 +11,7 @@
 #include <stdlib.h>
 
 #include <atomic>
+#include <mutex>
 #include <type_traits>
 
 #include "common.hpp"
@@ -56,6 +57,14 @@ struct GemmArgs {
     // linear (no K split): [tiles along N][M] maxima of |y| over each tile's columns, which
     // the tile kernel writes beside the f32 rows and requant_rows_wide_kernel reduces.
     float *row_absmax_parts;
+    // Weight-streaming kernel that quantizes the f32 activations xf32 itself, into stage_codes
+    // and stage_scales (which A and sa name too): M workgroups do, and count themselves in
+    // counter sync_slot; the others wait (at most spin_limit polls) until it reads stage_target.
+    int8_t *stage_codes;
+    float *stage_scales;
+    int sync_slot;
+    int spin_limit;
+    unsigned stage_target;
 };
 
 // LDS tiles are rows of BK bytes (BK/16 chunks of 16 bytes).  The chunk index
@@ -778,6 +787,100 @@ __global__ __launch_bounds__(256) void requant_rows_wide_kernel(const float *__r
             out[(n + 1024 * i) >> 2] = vtlhip::qdev::quant4(v[i], qp);
 }
 
+// Workgroup barrier that orders LDS traffic only: unlike __syncthreads() it does
+// not wait for outstanding global loads, so direct-to-LDS weight loads issued
+// earlier stay in flight across it.
+__device__ __forceinline__ void lds_barrier()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+// ---- activations quantized inside the weight-streaming launch ----------------
+//
+// A decode-shaped linear on f32 activations used to be two launches, the row quantizer and the
+// weight-streaming kernel; the first cost 3.2 us in front of a 12 us kernel, nearly all of it
+// launch latency.  Here one launch does both.  Its first M workgroups ("producers",
+// dispatched first) quantize one activation row each into the staging buffer and count
+// themselves in the slot's counter; the other workgroups start their weight stream, wait
+// until the counter has reached the value the host computed for this launch, and then read
+// codes and scales as they would after a quantizer launch (N = 14336, K = 4096: 14.4 against
+// 16.0 us with 8 rows, 16.8 against 18.8 us with 32).  Splitting a row's conversion over
+// several producers, or giving every XCD producers and a staging copy of its own (nothing
+// then leaves an L2), measured slower: both read the cold activations more often.
+//
+// Coherence.  The chip has eight L2 caches (one per XCD) that do not snoop each other, and a
+// release or acquire fence of device scope writes back or invalidates a whole L2: a few tenths
+// of a microsecond each, 40 us for the ~900 waves of such a launch (measured).  So no fence is
+// used.  Producers store codes and scales with device-scope stores, which go through their
+// L2 to memory, wait until those are acknowledged (s_waitcnt vmcnt(0), then the workgroup
+// barrier) and only then count themselves; the counter is touched with device-scope atomics
+// only, which are carried out at the memory side.  A waiting workgroup cannot hold a stale
+// copy of the staging buffer: every cache was invalidated when the launch began and nothing
+// reads the buffer before the count is complete (a workgroup that gives up waiting writes
+// the same values before it reads them), so its ordinary loads miss and fetch what the
+// producers wrote.
+//
+// The counter only ever grows: the host keeps, per slot, the sum of the producers of all
+// launches so far, so nothing needs clearing between launches; a launch recorded into a
+// graph would replay a stale target, so this form is not used while the stream is capturing.
+// There are 64 copies of the counter, 256 bytes apart; every producer adds to all of them (one
+// wave instruction) and a waiting workgroup polls one: 448 workgroups polling a single
+// address took longer than the quantizer launch this replaces.  The wait is bounded: after
+// spin_limit polls a workgroup quantizes all M rows itself (the same values into the same
+// places) and goes on, so the launch drains whatever the order in which workgroups start.
+// Launches that share a slot must not overlap.
+constexpr int kStageSlots = 16;
+constexpr int kStageCopies = 64;
+constexpr int kStageMaxK = 8192;
+__device__ unsigned g_stage_count[kStageSlots * kStageCopies * 64];
+
+__device__ __forceinline__ void stage_store(unsigned *p, unsigned v)
+{
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ void wait_memory_acknowledged()
+{
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+// One row of K floats (K % 4 == 0, K <= 8192) by a workgroup of NT threads: scale = absmax / 127,
+// codes as the row quantizer makes them, stored through to memory; a thread returns when its
+// stores are acknowledged.  `red` holds NT / 64 floats; the caller puts a barrier between two
+// calls.
+template <int NT>
+__device__ __forceinline__ void stage_quantize_row(const float *x, int K, int8_t *q, float *scale_out, float *red)
+{
+    constexpr int NV = kStageMaxK / 4 / NT;
+    const vtlhip::qdev::float4_t *xv = reinterpret_cast<const vtlhip::qdev::float4_t *>(x);
+    unsigned *qv = reinterpret_cast<unsigned *>(q);
+    const int nv = K >> 2;
+    vtlhip::qdev::float4_t v[NV];
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int idx = i * NT + (int)threadIdx.x;
+        v[i] = idx < nv ? xv[idx] : vtlhip::qdev::float4_t{0.f, 0.f, 0.f, 0.f};
+    }
+    float m = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NV; i++)
+        m = vtlhip::qdev::absmax4(m, v[i]);
+    m = vtlhip::qdev::block_max<NT>(m, red);
+    const float scale = m / 127.0f;
+    if (threadIdx.x == 0)
+        stage_store(reinterpret_cast<unsigned *>(scale_out), __float_as_uint(scale));
+    const vtlhip::qdev::QuantScale p = vtlhip::qdev::make_quant_scale(scale);
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int idx = i * NT + (int)threadIdx.x;
+        if (idx < nv)
+            stage_store(qv + idx, vtlhip::qdev::quant4(v[i], p));
+    }
+    wait_memory_acknowledged();
+}
+
 // Weight-streaming kernel for M <= 32 (decode-shaped linear): bound by reading
 // the weight matrix once, so the design goal is bytes in flight and long
 // contiguous reads, not MFMA rate.  (With more activation rows grid.y walks
@@ -797,9 +900,10 @@ __global__ __launch_bounds__(256) void requant_rows_wide_kernel(const float *__r
 // of absent rows re-read existing ones and their output columns are never
 // stored.  Requires K % 256 == 0; rows past N are clamped on load and masked
 // on store.
-template <int NWAVE, int STAGES, int XJ, bool F32OUT>
+template <int NWAVE, int STAGES, int XJ, bool F32OUT, bool STAGEQ = false>
 __global__ __launch_bounds__(64 * NWAVE) void linear_skinny_kernel(const GemmArgs g)
 {
+    static_assert(!STAGEQ || STAGES == 2, "the staged form counts its first loads for a ring of two slots");
     constexpr int BK = 256;
     constexpr int WCHUNK = 32 * BK;              // 8 KiB of weights per slot
     constexpr int XROWS = 8 * XJ;
@@ -811,7 +915,22 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_skinny_kernel(const GemmArg
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int M = g.M, N = g.N, K = g.K;
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-    const int n0 = blockIdx.x * 32;
+    __shared__ float s_red[NWAVE];
+    __shared__ int s_ready;
+    int bx = blockIdx.x;
+    unsigned *const counter = g_stage_count + g.sync_slot * (kStageCopies * 64);
+    if constexpr (STAGEQ) {
+        if (bx < M) {   // producer: one activation row, then gone
+            stage_quantize_row<64 * NWAVE>(g.xf32 + (int64_t)bx * K, K, g.stage_codes + (int64_t)bx * K,
+                                           g.stage_scales + bx, s_red);
+            __syncthreads();   // every thread's share of the row is in memory
+            if (tid < kStageCopies)
+                __hip_atomic_fetch_add(counter + tid * 64, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return;
+        }
+        bx -= M;
+    }
+    const int n0 = bx * 32;
     const int m0 = blockIdx.y * 32;   // more than 32 activation rows: one block of 32 per grid row
     char *ring = smem + w * (STAGES * SLOT);
 
@@ -838,16 +957,23 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_skinny_kernel(const GemmArg
         const int lc = (lane & 15) ^ (row & 15);
         px[j] = g.A + (int64_t)min(m0 + row, M - 1) * K + (int64_t)kc_begin * BK + lc * 16;
     }
-    auto issue = [&](int c, int st) {
+    auto issue_w = [&](int c, int st) {
         char *sw_ = ring + st * SLOT;
-        char *sx_ = sw_ + WCHUNK;
         const int64_t ko = (int64_t)c * BK;
 #pragma unroll
         for (int j = 0; j < WLOADS; j++)
             __builtin_amdgcn_global_load_lds(VTL_GPTR(pw[j] + ko), VTL_LPTR(sw_ + j * 1024), 16, 0, 0);
+    };
+    auto issue_x = [&](int c, int st) {
+        char *sx_ = ring + st * SLOT + WCHUNK;
+        const int64_t ko = (int64_t)c * BK;
 #pragma unroll
         for (int j = 0; j < XLOADS; j++)
             __builtin_amdgcn_global_load_lds(VTL_GPTR(px[j] + ko), VTL_LPTR(sx_ + j * 1024), 16, 0, 0);
+    };
+    auto issue = [&](int c, int st) {
+        issue_w(c, st);
+        issue_x(c, st);
     };
 
     v16i acc0, acc1;
@@ -875,7 +1001,8 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_skinny_kernel(const GemmArg
         for (int it = 0; it < ITEMS; it++) {
             const int item = tid + it * 64 * NWAVE;
             const int m = m0 + (item >> 3), n = n0 + (item & 7) * 4;
-            e_sa[it] = m < M ? g.sa[(int64_t)m * g.sa_stride] : 0.0f;
+            if constexpr (!STAGEQ)
+                e_sa[it] = m < M ? g.sa[(int64_t)m * g.sa_stride] : 0.0f;
 #pragma unroll
             for (int k = 0; k < 4; k++) {
                 const bool in = m < M && n + k < N;
@@ -884,13 +1011,63 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_skinny_kernel(const GemmArg
             }
         }
     }
+    if constexpr (STAGEQ) {
+        // the weights of every ring slot are under way while the activations are being made
 #pragma unroll
-    for (int st = 0; st < STAGES - 1; st++)
-        if (st < KC)
-            issue(st, st);
+        for (int st = 0; st < STAGES; st++)
+            if (st < KC)
+                issue_w(st, st);
+        if (tid == 0) {
+            int seen = 0;
+            const unsigned *mine = counter + (bx % kStageCopies) * 64;
+            for (int spin = 0;; spin++) {
+                const unsigned now = __hip_atomic_load(mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if ((int)(now - g.stage_target) >= 0) {
+                    seen = 1;
+                    break;
+                }
+                if (spin >= g.spin_limit)
+                    break;
+                __builtin_amdgcn_s_sleep(1);
+            }
+            s_ready = seen;
+        }
+        lds_barrier();
+        if (!s_ready) {   // not seen in time: this workgroup makes the rows itself
+            for (int r = 0; r < M; r++) {
+                stage_quantize_row<64 * NWAVE>(g.xf32 + (int64_t)r * K, K, g.stage_codes + (int64_t)r * K,
+                                               g.stage_scales + r, s_red);
+                __syncthreads();
+            }
+        }
+        asm volatile("" ::: "memory");   // the loads below stay below
+        if constexpr (F32OUT) {
+#pragma unroll
+            for (int it = 0; it < ITEMS; it++) {
+                const int m = m0 + ((tid + it * 64 * NWAVE) >> 3);
+                e_sa[it] = m < M ? g.sa[m] : 0.0f;
+            }
+        }
+#pragma unroll
+        for (int st = 0; st < STAGES; st++)
+            if (st < KC)
+                issue_x(st, st);
+    } else {
+#pragma unroll
+        for (int st = 0; st < STAGES - 1; st++)
+            if (st < KC)
+                issue(st, st);
+    }
     int st_c = 0, st_l = STAGES - 1;
     for (int c = 0; c < KC; c++) {
-        if (c + STAGES - 1 < KC) {
+        if (STAGEQ && c == 0) {
+            // Both slots were filled above, the weight loads first (W0 W1 X0 X1): chunk 0 is
+            // there when only X1 is outstanding.
+            if (KC > 1)
+                wait_vmcnt<XLOADS>();
+            else
+                wait_vmcnt<0>();
+        } else if (c + STAGES - 1 < KC) {
             issue(c + STAGES - 1, st_l);
             wait_vmcnt<(STAGES - 1) * LOADS>();  // chunk c has landed
         } else {
@@ -978,16 +1155,6 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_skinny_kernel(const GemmArg
             }
         }
     }
-}
-
-// Workgroup barrier that orders LDS traffic only: unlike __syncthreads() it does
-// not wait for outstanding global loads, so direct-to-LDS weight loads issued
-// earlier stay in flight across it.
-__device__ __forceinline__ void lds_barrier()
-{
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
 }
 
 // Sum of an int over the 64 lanes of a wave, the same value returned to every
@@ -1710,24 +1877,96 @@ void choose_config(int M, int N, int K, int &best_idx, int &best_splits)
     }
 }
 
-template <int NWAVE, int STAGES, int XJ, bool F32OUT>
+template <int NWAVE, int STAGES, int XJ, bool F32OUT, bool STAGEQ = false>
 int launch_skinny_cfg(const GemmArgs &g, hipStream_t st)
 {
     constexpr int lds = NWAVE * STAGES * (8192 + XJ * 2048);
     static_assert(lds >= NWAVE * 4096, "room for the partial tiles");
     static PerDevice<DoneFlag> done_flag;
     DoneFlag &done = done_flag.get();
-    const dim3 grid((unsigned)((g.N + 31) / 32), (unsigned)((g.M + 31) / 32));
+    // STAGEQ: M <= 32, and in front the workgroups that quantize the activation rows
+    const dim3 grid((unsigned)((g.N + 31) / 32 + (STAGEQ ? g.M : 0)),
+                    STAGEQ ? 1u : (unsigned)((g.M + 31) / 32));
     if (grid.y > 65535)
         return VTL_HIP_ERR_UNSUPPORTED;
     if (!done.load(std::memory_order_acquire)) {
-        VTL_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(linear_skinny_kernel<NWAVE, STAGES, XJ, F32OUT>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        VTL_HIP_TRY(hipFuncSetAttribute(
+            reinterpret_cast<const void *>(linear_skinny_kernel<NWAVE, STAGES, XJ, F32OUT, STAGEQ>),
+            hipFuncAttributeMaxDynamicSharedMemorySize, lds));
         done.store(true, std::memory_order_release);
     }
-    hipLaunchKernelGGL((linear_skinny_kernel<NWAVE, STAGES, XJ, F32OUT>), grid, dim3(64 * NWAVE), lds, st, g);
+    hipLaunchKernelGGL((linear_skinny_kernel<NWAVE, STAGES, XJ, F32OUT, STAGEQ>), grid, dim3(64 * NWAVE), lds, st, g);
     return check_launch("linear_skinny_kernel");
 }
+
+// The three instances of the kernel that quantizes the activations itself, by row count.
+inline int launch_skinny_staged_cfg(const GemmArgs &g, hipStream_t st)
+{
+    if (g.M <= 8)
+        return launch_skinny_cfg<2, 2, 1, true, true>(g, st);
+    if (g.M <= 16)
+        return launch_skinny_cfg<2, 2, 2, true, true>(g, st);
+    return launch_skinny_cfg<2, 2, 4, true, true>(g, st);
+}
+
+// Host side of the launch that quantizes the activations itself.  Its workgroups meet on a
+// counter that only grows, so the host has to know what every earlier launch added to it and
+// launches that share a counter must run one after the other: each stream gets a counter of
+// its own (the first kStageSlots streams that ask, per device, for as long as the process
+// lives; a stream handle that is reused inherits its predecessor's counter, which is as good),
+// and the value it will reach is kept beside it.  No counter is handed out while the stream is
+// being captured (a replay would wait for a value that was reached long ago), nor when the
+// capture state cannot be queried.
+struct StageCounters {
+    std::mutex lock;
+    hipStream_t stream[kStageSlots] = {};
+    bool taken[kStageSlots] = {};
+    unsigned counted[kStageSlots] = {};
+};
+
+inline int stage_counter_of(StageCounters &c, hipStream_t st)
+{
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &capturing) != hipSuccess) {
+        (void)hipGetLastError();
+        return -1;
+    }
+    if (capturing != hipStreamCaptureStatusNone)
+        return -1;
+    for (int i = 0; i < kStageSlots; i++)
+        if (c.taken[i] && c.stream[i] == st)
+            return i;
+    for (int i = 0; i < kStageSlots; i++)
+        if (!c.taken[i]) {
+            c.taken[i] = true;
+            c.stream[i] = st;
+            return i;
+        }
+    return -1;
+}
+
+// The weight-streaming launch that quantizes the f32 activations g.xf32 itself, into
+// g.stage_codes / g.stage_scales (which g.A / g.sa name too).  M <= 32, K <= kStageMaxK.
+// `launched` is false when the stream has no counter: nothing was enqueued then and the
+// caller takes the two-launch path.
+inline int launch_skinny_staged(GemmArgs g, hipStream_t st, bool &launched)
+{
+    static PerDevice<StageCounters> counters;
+    StageCounters &c = counters.get();
+    std::lock_guard<std::mutex> hold(c.lock);
+    const int slot = stage_counter_of(c, st);
+    launched = slot >= 0;
+    if (!launched)
+        return VTL_HIP_OK;
+    g.sync_slot = slot;
+    g.spin_limit = tuning().stage_spin;
+    g.stage_target = c.counted[slot] + (unsigned)g.M;
+    const int rc = launch_skinny_staged_cfg(g, st);
+    if (rc == VTL_HIP_OK)
+        c.counted[slot] = g.stage_target;
+    return rc;
+}
+
 
 // nwave: K ranges (waves) per workgroup.  Two waves and two ring slots measured best for the
 // decode shapes (M <= 32 against thousands of weight rows): the small LDS footprint keeps every
@@ -2093,6 +2332,7 @@ int vtl_hip_gemm_tile_choice(int M, int N, int K, int *config_index, int *tile_m
     return VTL_HIP_OK;
 }
 
+
 size_t vtl_hip_linear_f32_dynquant_workspace(int M, int K)
 {
     if (M <= 0 || K <= 0)
@@ -2130,6 +2370,9 @@ int vtl_hip_linear_f32_dynquant(const float *X, const int8_t *Wq, const float *s
         GemmArgs g{nullptr, Wq, Y, nullptr, sw, bias, M, N, K, 1, 1, relu ? 1 : 0, 1, nullptr, X, 0};
         return launch_gemv_rows<true, true>(g, current_stream());
     }
+    const bool staged = M <= 32 && N >= 2048 && K % 256 == 0 && K <= kStageMaxK && aligned16(X) && aligned16(Wq) &&
+                        tuning().gemm_config < 0 && !tuning().no_fused_decode &&
+                        !(gemv_rows_applies(X, Wq, M, N, K) && gemv_rows_faster(M, N, K));
     if (!workspace) {   // no caller scratch: stage in the library's own buffer
         workspace = vtlhip::library_workspace(vtl_hip_linear_f32_dynquant_workspace(M, K), 1);
         if (!workspace)
@@ -2138,6 +2381,17 @@ int vtl_hip_linear_f32_dynquant(const float *X, const int8_t *Wq, const float *s
     int8_t *xq = reinterpret_cast<int8_t *>(workspace);
     const size_t codes = (((size_t)M * (size_t)K) + 255) & ~(size_t)255;
     float *sx = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + codes);
+    if (staged) {
+        // a few tokens against thousands of weight rows: quantized inside the weight-streaming
+        // launch (N = 14336, K = 4096, M = 8: 14.4 us against 16.0 us)
+        GemmArgs g{xq, Wq, Y, sx, sw, bias, M, N, K, 1, 1, relu ? 1 : 0, 1, nullptr, X, 0};
+        g.stage_codes = xq;
+        g.stage_scales = sx;
+        bool launched = false;
+        st = launch_skinny_staged(g, current_stream(), launched);
+        if (launched || st != VTL_HIP_OK)
+            return st;
+    }
     st = launch_quantize_rows(X, M, K, xq, sx, current_stream());
     if (st != VTL_HIP_OK)
         return st;

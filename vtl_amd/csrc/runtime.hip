@@ -70,6 +70,9 @@ static const Tuning *read_tuning(bool force)
     t->no_fused_requant = flag("VTL_HIP_NO_FUSED_REQUANT");
     t->requant_wide = number("VTL_HIP_REQUANT_WIDE", 0);
     t->no_fused_decode = flag("VTL_HIP_NO_FUSED_DECODE");
+    t->stage_spin = number("VTL_HIP_STAGE_SPIN", 4096);
+    if (t->stage_spin < 0 || t->stage_spin > (1 << 20))
+        t->stage_spin = 4096;
     t->skinny_tiled = number("VTL_HIP_SKINNY_TILED", -1);
     t->skinny_waves = number("VTL_HIP_SKINNY_WAVES", 4);
     t->matmul_tile = number("VTL_HIP_MATMUL_TILE", 0);
