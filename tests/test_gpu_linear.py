@@ -357,6 +357,50 @@ def test_decode_launch_counters_are_per_stream_and_run_out_gracefully(hip):
         SW.release()
 
 
+def test_decode_launches_on_two_streams_may_overlap(hip):
+    """Two streams, a staging buffer and a counter each: calls are enqueued on both without
+    waiting in between, so the launches are free to run at the same time, and each must wait
+    for its own rows only."""
+    hiprt = C.CDLL("libamdhip64.so")
+    n, k = 14336, 4096
+    rng = np.random.Generator(np.random.Philox(79))
+    w = rng.integers(-127, 128, (n, k), dtype=np.int8)
+    sw = (rng.uniform(0.5, 1.5, n) * 1e-3).astype(np.float32)
+    W, SW = dev(w), dev(sw)
+    lanes = []
+    try:
+        for i, m in enumerate((8, 32)):
+            st = C.c_void_p()
+            assert hiprt.hipStreamCreate(C.byref(st)) == 0
+            need = int(capi.lib().vtl_hip_linear_f32_dynquant_workspace(m, k))
+            xs = [rng.standard_normal((m, k), dtype=np.float32) * np.float32(j + 1 + 3 * i) for j in range(3)]
+            lanes.append({"stream": st, "m": m, "ws": HipTensor.empty([need], np.uint8), "xs": xs,
+                          "X": [dev(x) for x in xs], "Y": [HipTensor.empty([m, n], np.float32) for _ in xs],
+                          "want": [oracle.linear_f32_dynquant(x, w, sw, None, threads=CPU_THREADS) for x in xs]})
+        for rnd in range(4):
+            for j in range(3):
+                for ln in lanes:                    # alternate between the streams, no waiting
+                    capi.call("vtl_hip_set_stream", ln["stream"])
+                    capi.call("vtl_hip_linear_f32_dynquant", ln["X"][j].ptr, W.ptr, SW.ptr, None, ln["Y"][j].ptr,
+                              ln["m"], n, k, 0, ln["ws"].ptr, ln["ws"].size)
+            for ln in lanes:
+                capi.call("vtl_hip_set_stream", ln["stream"])
+                capi.call("vtl_hip_sync")
+            for ln in lanes:
+                for j in range(3):
+                    assert np.array_equal(ln["Y"][j].cpu(), ln["want"][j]), (rnd, ln["m"], j)
+                    capi.call("vtl_hip_memset", ln["Y"][j].ptr, 0, ln["m"] * n * 4)
+    finally:
+        capi.call("vtl_hip_set_stream", None)
+        capi.call("vtl_hip_sync")
+        for ln in lanes:
+            hiprt.hipStreamDestroy(ln["stream"])
+            for t in [ln["ws"], *ln["X"], *ln["Y"]]:
+                t.release()
+        W.release()
+        SW.release()
+
+
 def test_decode_launch_is_replaced_by_two_launches_under_stream_capture(hip):
     """A graph replays the kernel arguments it recorded, and the launch that quantizes its own
     rows waits for a counter value that is new on every call: under capture the library records

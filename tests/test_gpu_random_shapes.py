@@ -71,6 +71,39 @@ def test_random_shapes_linear_with_quantization_on_the_fly(hip, block):
                 h.release()
 
 
+@pytest.mark.parametrize("block", range(3))
+def test_random_decode_shapes_quantized_inside_the_launch(hip, block):
+    """2 to 32 tokens, thousands of weight rows, K any multiple of 256 up to 8192: the shapes
+    of the launch whose first workgroups quantize the tokens for the others.  Row magnitudes
+    spread over 17 decades, zero rows, staging buffers that come and go between calls (so a
+    later call finds other codes at an address an earlier one used)."""
+    rng = np.random.Generator(np.random.Philox(2500 + block))
+    for _ in range(16):
+        m = int(rng.integers(2, 33))
+        n = int(rng.integers(2048, 20001))
+        k = 256 * int(rng.integers(1, 33))
+        while m * n * k > 1.5e9:
+            n = max(2048, n // 2)
+            k = max(256, (k // 2) & ~255)
+        x = (rng.standard_normal((m, k)) * np.exp(rng.uniform(-20, 20, (m, 1)))).astype(np.float32)
+        if rng.random() < 0.4:
+            x[int(rng.integers(0, m))] = 0.0
+        w = rng.integers(-127, 128, (n, k), dtype=np.int8)
+        sw = (rng.uniform(0.5, 1.5, n) * 1e-3).astype(np.float32)
+        bias = rng.standard_normal(n).astype(np.float32) if rng.random() < 0.7 else None
+        relu = bool(rng.integers(0, 2))
+        X, W, SW = dev(x), dev(w), dev(sw)
+        BI = dev(bias) if bias is not None else None
+        want = oracle.linear_f32_dynquant(x, w, sw, bias, relu=relu, threads=CPU_THREADS)
+        for _rep in range(2):
+            y = linear_f32_dynquant_hip(X, W, SW, BI, relu=relu)
+            assert np.array_equal(y.cpu(), want), (m, n, k)
+            y.release()
+        for h in (X, W, SW, BI):
+            if h is not None:
+                h.release()
+
+
 @pytest.mark.parametrize("block", range(4))
 def test_random_shapes_quantize_dequantize_absmax(hip, block):
     """Row counts and row lengths drawn blindly (odd lengths, single rows and columns,

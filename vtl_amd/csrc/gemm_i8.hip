@@ -106,12 +106,6 @@ __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int bloc
     tile_n = (pid % group_size) / gm;
 }
 
-// Epilogue shared by the tiled kernels.  Accumulator register r of lane l of a
-// 32x32 MFMA tile holds row 8*(r/4) + 4*(l/32) + r%4, column l%32.  The scale
-// and bias slices of the block tile are staged in LDS (free once the K loop is
-// over); every output element is
-//     y = fl(fl(f32(acc) * fl(sa*sw)) + bias), then ReLU,
-// evaluated in that order with separately rounded operations.
 // Scales and bias of a block tile, fetched by the threads of the workgroup before the K loop
 // (thread t takes rows / columns t, t + NT, ...) and put into LDS by the epilogue: read only
 // then, they add a memory latency to the end of every workgroup.  Used by the 256x256 tile
@@ -143,6 +137,12 @@ __device__ __forceinline__ void fetch_scales(EpilogueScales<BM, BN, NT> &e, cons
     }
 }
 
+// Epilogue shared by the tiled kernels.  Accumulator register r of lane l of a
+// 32x32 MFMA tile holds row 8*(r/4) + 4*(l/32) + r%4, column l%32.  The scale
+// and bias slices of the block tile are staged in LDS (free once the K loop is
+// over); every output element is
+//     y = fl(fl(f32(acc) * fl(sa*sw)) + bias), then ReLU,
+// evaluated in that order with separately rounded operations.
 template <int BM, int BN, int WM, int WN, bool F32OUT, bool EDGE, int NT, bool ROWMAX = false>
 __device__ __forceinline__ void epilogue(v16i (&acc)[WM / 32][WN / 32], const GemmArgs &g, int m0, int n0,
                                          int wr, int wc, char *smem, const EpilogueScales<BM, BN, NT> &pre)
