@@ -164,8 +164,8 @@ int vtl_hip_linear_i8_requant(const int8_t *A, const float *sa, int sa_per_row,
  * staging buffers, autograd_cuda/device_session.v:13-24); NULL (with size 0)
  * makes the library stage in a buffer of its own, one per device, grown on
  * demand.  Calls that may overlap on a device (several streams) need a
- * workspace each.  For 2 to 32 rows against at least 2048 weight rows
- * (K % 256 == 0, K <= 8192) quantizer and linear are one launch whose
+ * workspace each.  For 2 to 32 rows with K % 256 == 0 and K <= 8192 (most such
+ * shapes from 128 weight rows on) quantizer and linear are one launch whose
  * workgroups meet on a device counter that the library keeps per stream, for
  * the first 16 streams that make such a call; calls on further streams, and
  * calls made while the stream is being captured into a graph, are two

@@ -274,8 +274,10 @@ def test_few_token_fused_decode_equals_two_launch_path(hip, mnk, knobs):
         h.release()
 
 
-@pytest.mark.parametrize("mnk", [(2, 2048, 256), (8, 14336, 4096), (8, 2077, 1280), (9, 3001, 512), (16, 2048, 8192),
-                                 (17, 4096, 2048), (31, 2050, 4096), (32, 14336, 4096)])
+@pytest.mark.parametrize("mnk", [(2, 2048, 256), (8, 14336, 4096), (8, 2077, 1280), (9, 3001, 512), (16, 12300, 8192),
+                                 (17, 4096, 2048), (31, 2050, 4096), (32, 14336, 4096), (3, 14336, 4096),
+                                 # fewer than 2048 weight rows: the four-wave form of the kernel
+                                 (12, 512, 1024), (32, 1920, 2048), (5, 128, 4096), (16, 1000, 4096), (8, 300, 2048)])
 def test_decode_launch_that_quantizes_its_rows_equals_two_launch_path(hip, mnk, knobs):
     """2 to 32 tokens against thousands of weight rows: one launch whose first workgroups
     quantize the rows while the others wait for them.  Same bits as quantizer + linear and as

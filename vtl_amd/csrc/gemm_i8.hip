@@ -1899,9 +1899,35 @@ int launch_skinny_cfg(const GemmArgs &g, hipStream_t st)
     return check_launch("linear_skinny_kernel");
 }
 
-// The three instances of the kernel that quantizes the activations itself, by row count.
+// Where the launch that quantizes the activations itself beats quantizer + linear, from a sweep
+// of N = 128 .. 14336, K = 1024 .. 8192, M = 2 .. 32 (weights cached and from HBM): with
+// thousands of weight rows whenever K <= 4096 (0.3 to 2.2 us of 6 to 19 us), with K = 8192 only
+// from about 12288 rows on (with fewer rows the wait for 8192-element rows is not hidden: 14.4
+// against 12.9 us at 8 x 4096 x 8192); below 2048 weight rows, where the linear is the four-wave
+// form, for K = 1024 .. 4096 (7.3 -> 5.0 us at 16 x 512 x 1024, 8.1 -> 7.2 us at 16 x 1024 x 4096).
+// `few_token_kernel`: the matrix-vector kernel for 2 to 8 rows (behind a quantizer launch)
+// would take the product; it keeps it except below 2048 rows and on the largest matrices.
+inline bool stage_inside_launch_faster(int M, int N, int K, bool few_token_kernel)
+{
+    if (M > 32 || K % 256 != 0 || K > kStageMaxK)
+        return false;
+    if (N < 2048)   // (3 or 4 rows of more than 2048 elements stay with the matrix-vector kernel: within 0.5 us either way)
+        return N >= 128 && K >= 1024 && K <= 4096 && (M >= 5 || K <= 2048);
+    if (few_token_kernel && !(N >= 12288 && K <= 4096))
+        return false;
+    return K <= 4096 || N >= 12288;
+}
+
+// The instances of the kernel that quantizes the activations itself, by row count.
 inline int launch_skinny_staged_cfg(const GemmArgs &g, hipStream_t st)
 {
+    if (g.N < 2048) {   // few row blocks: K over four waves, as launch_skinny does for them
+        if (g.M <= 8)
+            return launch_skinny_cfg<4, 2, 1, true, true>(g, st);
+        if (g.M <= 16)
+            return launch_skinny_cfg<4, 2, 2, true, true>(g, st);
+        return launch_skinny_cfg<4, 2, 4, true, true>(g, st);
+    }
     if (g.M <= 8)
         return launch_skinny_cfg<2, 2, 1, true, true>(g, st);
     if (g.M <= 16)
@@ -2370,9 +2396,8 @@ int vtl_hip_linear_f32_dynquant(const float *X, const int8_t *Wq, const float *s
         GemmArgs g{nullptr, Wq, Y, nullptr, sw, bias, M, N, K, 1, 1, relu ? 1 : 0, 1, nullptr, X, 0};
         return launch_gemv_rows<true, true>(g, current_stream());
     }
-    const bool staged = M <= 32 && N >= 2048 && K % 256 == 0 && K <= kStageMaxK && aligned16(X) && aligned16(Wq) &&
-                        tuning().gemm_config < 0 && !tuning().no_fused_decode &&
-                        !(gemv_rows_applies(X, Wq, M, N, K) && gemv_rows_faster(M, N, K));
+    const bool staged = stage_inside_launch_faster(M, N, K, gemv_rows_applies(X, Wq, M, N, K) && gemv_rows_faster(M, N, K)) &&
+                        aligned16(X) && aligned16(Wq) && tuning().gemm_config < 0 && !tuning().no_fused_decode;
     if (!workspace) {   // no caller scratch: stage in the library's own buffer
         workspace = vtlhip::library_workspace(vtl_hip_linear_f32_dynquant_workspace(M, K), 1);
         if (!workspace)
