@@ -318,12 +318,14 @@ __device__ __attribute__((aligned(16))) int8_t g_zero_chunk[16];
 // barrier sits before the last k-step of a tile so that its latency and the
 // first operand reads of the next tile hide behind that step's MFMAs, and the
 // loads that refill the freed stage are issued a few at a time between MFMAs.
-// Requires K % BK == 0, or with EDGE K % 16 == 0: then the chunks of the last
-// tile that lie past K are loaded as zeros, rows past M / N are clamped on load
-// and masked on store.
-template <int BM, int BN, int BK, int NSTAGE, int WR, int WC, bool F32OUT, bool EDGE, bool SPLIT, bool ROWMAX = false>
+// Requires K % BK == 0; with EDGE rows past M / N are clamped on load and masked
+// on store; with KTAIL (and EDGE) K % 16 == 0 is enough: the chunks of the last
+// tile that lie past K are loaded as zeros.
+template <int BM, int BN, int BK, int NSTAGE, int WR, int WC, bool F32OUT, bool EDGE, bool SPLIT, bool ROWMAX = false,
+          bool KTAIL = false>
 __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArgs g)
 {
+    static_assert(EDGE || !KTAIL, "a partial last K tile is handled by the kernels that also clamp rows");
     constexpr int NW = WR * WC, NT = 64 * NW;
     constexpr int WM = BM / WR, WN = BN / WC, TM = WM / 32, TN = WN / 32;
     constexpr int CPR = BK / 16;   // 16-byte chunks per tile row
@@ -347,7 +349,7 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArg
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int wr = w / WC, wc = w % WC;
-    const int kt_all = EDGE ? (K + BK - 1) / BK : K / BK;  // EDGE: the last tile may be partial in K
+    const int kt_all = KTAIL ? (K + BK - 1) / BK : K / BK;  // KTAIL: the last tile may be partial in K
     const int kt_begin = SPLIT ? (int)((int64_t)kt_all * split / nsplit) : 0;
     const int kt_end = SPLIT ? (int)((int64_t)kt_all * (split + 1) / nsplit) : kt_all;
 
@@ -368,18 +370,27 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArg
         pb[0] = g.Bt + (int64_t)(n0 + lrow) * K + lc * 16;
     }
     const int64_t jstride = (int64_t)RPI * NW * K;
+    // The address of the zero chunk, made opaque to the compiler: left to itself it fetches the
+    // address from the global offset table inside the K loop and waits for that scalar load in
+    // every iteration (2.3 to 3 us of a 14 us launch with ragged M or N).
+    const int8_t *zero_chunk = g_zero_chunk;
+    if constexpr (KTAIL)
+        asm volatile("" : "+s"(zero_chunk));
     // Global source of load d (A rows first, then B) of the tile at K offset ko.
-    // With EDGE, a lane whose 16-byte chunk lies past K reads zeros instead
-    // (K % 16 == 0, so a chunk is inside or outside as a whole).
+    // With KTAIL, a lane whose 16-byte chunk lies past K reads zeros instead
+    // (K % 16 == 0, so a chunk is inside or outside as a whole).  That costs a
+    // compare per tile and two selects per load and lane in the K loop (1.5 to
+    // 2 us of a 12 us launch), so kernels for ragged M or N with a whole number
+    // of K tiles are built without it.
     auto source = [&](int d, int64_t ko) -> const int8_t * {
         const int8_t *p;
         if (d < A_PW)
             p = EDGE ? pa[EDGE ? d : 0] + ko : pa[0] + ko + d * jstride;
         else
             p = EDGE ? pb[EDGE ? d - A_PW : 0] + ko : pb[0] + ko + (d - A_PW) * jstride;
-        if constexpr (EDGE) {
+        if constexpr (KTAIL) {
             if (ko + lc * 16 >= K)
-                p = g_zero_chunk;
+                p = zero_chunk;
         }
         return p;
     };
@@ -1695,10 +1706,12 @@ int launch_dma(GemmArgs g, int splits, hipStream_t st)
         if (!g.partials)
             return vtlhip::workspace_status();
     }
-    static PerDevice<DoneFlag> done_flags[8];
-    DoneFlag *done[8] = {&done_flags[0].get(), &done_flags[1].get(), &done_flags[2].get(), &done_flags[3].get(),
-                     &done_flags[4].get(), &done_flags[5].get(), &done_flags[6].get(), &done_flags[7].get()};
-    const bool edge = (g.M % BM) || (g.N % BN) || (g.K % BK);
+    static PerDevice<DoneFlag> done_flags[12];
+    DoneFlag *done[12];
+    for (int i = 0; i < 12; i++)
+        done[i] = &done_flags[i].get();
+    const bool ktail = (g.K % BK) != 0;
+    const bool edge = (g.M % BM) || (g.N % BN) || ktail;
     g.cached_out = tiles <= 256 ? 1 : 0;  // one round of workgroups
     int rc;
     if (requant && splits == 1) {
@@ -1724,7 +1737,10 @@ int launch_dma(GemmArgs g, int splits, hipStream_t st)
                 GemmArgs gf = g;
                 gf.out = g.out ? g.out : reinterpret_cast<void *>(ws);
                 gf.row_absmax_parts = reinterpret_cast<float *>(ws + plane);
-                if (edge)
+                if (ktail)
+                    rc = launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, true, true, false, true, true>,
+                                         *done[8], lds, tiles, 64 * WR * WC, gf, st, "gemm_i8_dma_kernel");
+                else if (edge)
                     rc = launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, true, true, false, true>,
                                          *done[6], lds, tiles, 64 * WR * WC, gf, st, "gemm_i8_dma_kernel");
                 else
@@ -1744,7 +1760,10 @@ int launch_dma(GemmArgs g, int splits, hipStream_t st)
         // the int32 sums of the whole K go to the scratch plane the row kernel reads
         GemmArgs gi = g;
         gi.out = g.partials;
-        if (edge)
+        if (ktail)
+            rc = launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, false, true, false, false, true>,
+                                 *done[9], lds, tiles, 64 * WR * WC, gi, st, "gemm_i8_dma_kernel");
+        else if (edge)
             rc = launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, false, true, false>, *done[4], lds,
                                  tiles, 64 * WR * WC, gi, st, "gemm_i8_dma_kernel");
         else
@@ -1753,12 +1772,18 @@ int launch_dma(GemmArgs g, int splits, hipStream_t st)
         return rc != VTL_HIP_OK ? rc : launch_finalize_requant(g, st);
     }
     // the partial sums of a split launch are int32 whatever the final type is
-    if (splits > 1 && edge)
+    if (splits > 1 && ktail)
+        rc = launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, false, true, true, false, true>, *done[10],
+                             lds, tiles * splits, 64 * WR * WC, g, st, "gemm_i8_dma_kernel");
+    else if (splits > 1 && edge)
         rc = launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, false, true, true>, *done[0], lds,
                              tiles * splits, 64 * WR * WC, g, st, "gemm_i8_dma_kernel");
     else if (splits > 1)
         rc = launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, false, false, true>, *done[1], lds,
                              tiles * splits, 64 * WR * WC, g, st, "gemm_i8_dma_kernel");
+    else if (ktail)
+        rc = launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, F32OUT, true, false, false, true>,
+                             *done[11], lds, tiles, 64 * WR * WC, g, st, "gemm_i8_dma_kernel");
     else if (edge)
         rc = launch_with_lds(gemm_i8_dma_kernel<BM, BN, BK, NSTAGE, WR, WC, F32OUT, true, false>, *done[2], lds,
                              tiles, 64 * WR * WC, g, st, "gemm_i8_dma_kernel");
