@@ -347,7 +347,8 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArg
     tile_of_block((M + BM - 1) / BM, (N + BN - 1) / BN, SPLIT ? (int)(blockIdx.x / nsplit) : (int)blockIdx.x,
                   tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // the wave's index: uniform, so kept in a scalar register
     const int wr = w / WC, wc = w % WC;
     const int kt_all = KTAIL ? (K + BK - 1) / BK : K / BK;  // KTAIL: the last tile may be partial in K
     const int kt_begin = SPLIT ? (int)((int64_t)kt_all * split / nsplit) : 0;
@@ -356,23 +357,28 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArg
     // ---- global -> LDS ----
     const int lrow = RPI * w + lane / CPR;                  // tile row of this lane for j = 0
     const int lc = (lane % CPR) ^ swizzle<BK>(lrow);        // logical chunk it fetches (same for all j)
-    const int8_t *pa[EDGE ? A_PW : 1];
-    const int8_t *pb[EDGE ? B_PW : 1];
+    // A load address is a uniform 64-bit part (operand, first row of the tile, K offset and,
+    // without EDGE, the rows of load j) plus the lane's 32-bit offset from that row (at most
+    // 255 rows of K <= 131072 bytes), which is the form the load instruction takes a scalar base
+    // and a vector offset for: no vector arithmetic per load in the K loop.  With EDGE the
+    // offsets differ per load, rows past M / N being clamped.
+    unsigned oa[EDGE ? A_PW : 1], ob[EDGE ? B_PW : 1];
     if constexpr (EDGE) {
 #pragma unroll
         for (int j = 0; j < A_PW; j++)
-            pa[j] = g.A + (int64_t)min(m0 + lrow + j * RPI * NW, M - 1) * K + lc * 16;
+            oa[j] = (unsigned)(min(m0 + lrow + j * RPI * NW, M - 1) - m0) * (unsigned)K + (unsigned)(lc * 16);
 #pragma unroll
         for (int j = 0; j < B_PW; j++)
-            pb[j] = g.Bt + (int64_t)min(n0 + lrow + j * RPI * NW, N - 1) * K + lc * 16;
+            ob[j] = (unsigned)(min(n0 + lrow + j * RPI * NW, N - 1) - n0) * (unsigned)K + (unsigned)(lc * 16);
     } else {
-        pa[0] = g.A + (int64_t)(m0 + lrow) * K + lc * 16;
-        pb[0] = g.Bt + (int64_t)(n0 + lrow) * K + lc * 16;
+        oa[0] = ob[0] = (unsigned)lrow * (unsigned)K + (unsigned)(lc * 16);
     }
+    const int8_t *const a0 = g.A + (int64_t)m0 * K;
+    const int8_t *const b0 = g.Bt + (int64_t)n0 * K;
     const int64_t jstride = (int64_t)RPI * NW * K;
     // The address of the zero chunk, made opaque to the compiler: left to itself it fetches the
     // address from the global offset table inside the K loop and waits for that scalar load in
-    // every iteration (2.3 to 3 us of a 14 us launch with ragged M or N).
+    // every iteration.
     const int8_t *zero_chunk = g_zero_chunk;
     if constexpr (KTAIL)
         asm volatile("" : "+s"(zero_chunk));
@@ -385,9 +391,9 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_i8_dma_kernel(const GemmArg
     auto source = [&](int d, int64_t ko) -> const int8_t * {
         const int8_t *p;
         if (d < A_PW)
-            p = EDGE ? pa[EDGE ? d : 0] + ko : pa[0] + ko + d * jstride;
+            p = (a0 + ko + (EDGE ? 0 : d * jstride)) + (uint64_t)oa[EDGE ? d : 0];
         else
-            p = EDGE ? pb[EDGE ? d - A_PW : 0] + ko : pb[0] + ko + (d - A_PW) * jstride;
+            p = (b0 + ko + (EDGE ? 0 : (d - A_PW) * jstride)) + (uint64_t)ob[EDGE ? d - A_PW : 0];
         if constexpr (KTAIL) {
             if (ko + lc * 16 >= K)
                 p = zero_chunk;
@@ -925,7 +931,8 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_skinny_kernel(const GemmArg
     static_assert((STAGES - 1) * LOADS <= 63, "vmcnt is a 6-bit counter");
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int M = g.M, N = g.N, K = g.K;
-    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform in a wave: a scalar, and with it the ring addresses
     __shared__ float s_red[NWAVE];
     __shared__ int s_ready;
     int bx = blockIdx.x;
@@ -1205,7 +1212,7 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_gemv_kernel(const GemmArgs 
     __shared__ __attribute__((aligned(16))) int8_t xq[DYNQ ? 1024 * KV : 16];
     const int N = g.N, K = g.K;
     const int kv = K >> 4;  // 16-byte pieces of a row
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     // rows are dealt out cyclically: wave i of W takes rows i, i + W, i + 2 W, ... so that at any
     // moment the waves of the chip read one contiguous stretch of the matrix
     const int64_t W = (int64_t)gridDim.x * NWAVE;
@@ -1386,7 +1393,7 @@ __global__ __launch_bounds__(512) void linear_gemv_rows_kernel(const GemmArgs g)
     __shared__ __attribute__((aligned(16))) int8_t xq[DYNQ ? MR * 1024 * KV : 16];
     const int M = g.M, N = g.N, K = g.K;
     const int kv = K >> 4;  // 16-byte pieces of a row
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int64_t W = (int64_t)gridDim.x * NWAVE;
     const int64_t r0 = (int64_t)blockIdx.x * NWAVE + w, r1 = N;
 
@@ -1593,7 +1600,7 @@ template <bool F32OUT, int NW, int U>
 __global__ __launch_bounds__(64 * NW) void gemm_i8_small_kernel(const GemmArgs g)
 {
     __shared__ int red[NW][16][64];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int tiles_n = (g.N + 31) / 32;
     const int m0 = (int)(blockIdx.x / tiles_n) * 32, n0 = (int)(blockIdx.x % tiles_n) * 32;
     const int r = lane & 31, half = lane >> 5;
