@@ -165,11 +165,12 @@ int vtl_hip_linear_i8_requant(const int8_t *A, const float *sa, int sa_per_row,
  * makes the library stage in a buffer of its own, one per device, grown on
  * demand.  Calls that may overlap on a device (several streams) need a
  * workspace each.  For 2 to 32 rows with K % 256 == 0 and K <= 8192 (most such
- * shapes from 128 weight rows on) quantizer and linear are one launch whose
- * workgroups meet on a device counter that the library keeps per stream, for
- * the first 16 streams that make such a call; calls on further streams, and
- * calls made while the stream is being captured into a graph, are two
- * launches with the same results. */
+ * shapes from 128 weight rows on) and a workspace that starts on a 128-byte
+ * boundary (anything vtl_hip_malloc returns), quantizer and linear are one
+ * launch whose workgroups meet on a device counter that the library keeps per
+ * stream, for the first 16 streams that make such a call; calls on further
+ * streams, and calls made while the stream is being captured into a graph,
+ * are two launches with the same results. */
 size_t vtl_hip_linear_f32_dynquant_workspace(int M, int K);
 int vtl_hip_linear_f32_dynquant(const float *X, const int8_t *Wq, const float *sw,
                                 const float *bias, float *Y, int M, int N, int K, int relu,

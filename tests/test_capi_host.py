@@ -83,8 +83,8 @@ def test_bad_arguments_return_status_not_abort():
 def test_dynquant_workspace_size():
     f = capi.lib().vtl_hip_linear_f32_dynquant_workspace
     assert f(0, 16) == 0 and f(4, 0) == 0
-    assert f(1, 4096) == 4096 + 4
-    assert f(3, 100) == 512 + 12           # codes rounded up to 256 bytes
+    assert f(1, 4096) == 4096 + 256
+    assert f(3, 100) == 512 + 256          # codes and scales each rounded up to 256 bytes
     assert f(256, 11008) == 256 * 11008 + 1024
 
 

@@ -324,6 +324,30 @@ def test_decode_launch_that_quantizes_its_rows_equals_two_launch_path(hip, mnk, 
         h.release()
 
 
+def test_decode_with_a_staging_buffer_that_starts_inside_a_cache_line(hip):
+    """The one-launch form needs the staging buffer to own its cache lines; a buffer that is
+    16-byte but not 128-byte aligned gets quantizer + linear, with the same bits, and what lies
+    in front of it in the same line is left alone."""
+    m, n, k = 8, 4096, 1024
+    rng = np.random.Generator(np.random.Philox(80))
+    x = rng.standard_normal((m, k), dtype=np.float32)
+    w = rng.integers(-127, 128, (n, k), dtype=np.int8)
+    sw = (rng.uniform(0.5, 1.5, n) * 1e-3).astype(np.float32)
+    X, W, SW = dev(x), dev(w), dev(sw)
+    Y = HipTensor.empty([m, n], np.float32)
+    need = int(capi.lib().vtl_hip_linear_f32_dynquant_workspace(m, k))
+    buf = HipTensor.from_host(np.full(need + 256, 0x5A, np.uint8))
+    want = oracle.linear_f32_dynquant(x, w, sw, None)
+    for shift in (16, 48, 112, 0):
+        capi.call("vtl_hip_linear_f32_dynquant", X.ptr, W.ptr, SW.ptr, None, Y.ptr, m, n, k, 0,
+                  C.c_void_p(int(buf.ptr) + shift), need)
+        assert np.array_equal(Y.cpu(), want), shift
+        host = buf.cpu()
+        assert (host[:shift] == 0x5A).all() and (host[shift + need:] == 0x5A).all(), shift
+    for t in (X, W, SW, Y, buf):
+        t.release()
+
+
 def test_decode_launch_counters_are_per_stream_and_run_out_gracefully(hip):
     """The workgroups of that launch meet on a counter the library keeps per stream (16 of
     them): calls that alternate between streams, and calls on more streams than there are

@@ -2395,9 +2395,11 @@ size_t vtl_hip_linear_f32_dynquant_workspace(int M, int K)
 {
     if (M <= 0 || K <= 0)
         return 0;
-    // int8 codes of X, rounded up to 256 bytes, then M row scales
+    // int8 codes of X, then M row scales, each rounded up to 256 bytes: a buffer of this size that
+    // starts on a cache line owns every line it touches (the launch that quantizes the rows
+    // itself relies on nothing else living in those lines)
     const size_t codes = (((size_t)M * (size_t)K) + 255) & ~(size_t)255;
-    return codes + (size_t)M * sizeof(float);
+    return codes + (((size_t)M * sizeof(float) + 255) & ~(size_t)255);
 }
 
 int vtl_hip_linear_f32_dynquant(const float *X, const int8_t *Wq, const float *sw, const float *bias,
@@ -2438,9 +2440,12 @@ int vtl_hip_linear_f32_dynquant(const float *X, const int8_t *Wq, const float *s
     int8_t *xq = reinterpret_cast<int8_t *>(workspace);
     const size_t codes = (((size_t)M * (size_t)K) + 255) & ~(size_t)255;
     float *sx = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + codes);
-    if (staged) {
-        // a few tokens against thousands of weight rows: quantized inside the weight-streaming
-        // launch (N = 14336, K = 4096, M = 8: 14.4 us against 16.0 us)
+    if (staged && (reinterpret_cast<uintptr_t>(workspace) & 127) == 0) {
+        // a few tokens: quantized inside the weight-streaming launch (N = 14336, K = 4096, M = 8:
+        // 14.4 us against 16.0 us).  Its workgroups read the staging buffer as soon as the rows
+        // are counted and rely on no cache holding an older copy of those lines, which holds
+        // when nothing else shares them: the buffer starts on a cache line (anything from
+        // vtl_hip_malloc does) and its size is a whole number of them.
         GemmArgs g{xq, Wq, Y, sx, sw, bias, M, N, K, 1, 1, relu ? 1 : 0, 1, nullptr, X, 0};
         g.stage_codes = xq;
         g.stage_scales = sx;
