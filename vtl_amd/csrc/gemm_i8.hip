@@ -1909,6 +1909,18 @@ void choose_config(int M, int N, int K, int &best_idx, int &best_splits)
     }
 }
 
+// Waves (K ranges) per workgroup for up to 32 rows against 2048 weight rows or more.  From a
+// sweep of M = 2 .. 32, N = 2048 .. 14336, K = 1024 .. 11008, cached and from HBM: four waves
+// up to 256 workgroups (N <= 8192: half the chip or less would otherwise run two waves each;
+// 12 x 2048 x 4096 5.9 -> 4.8 us, 16 x 4096 x 8192 9.1 -> 6.8 us) and whenever K >= 8192
+// (6 x 14336 x 8192 from HBM 26.4 -> 21.5 us); two waves for more workgroups with a shorter K,
+// where the smaller LDS footprint keeps every workgroup resident (24 x 11008 x 4096: 9.7 against
+// 10.6 us).  Mean regret against the best of both over the sweep 1.1 % cached, 2.1 % from HBM.
+inline int skinny_waves_few_rows(int N, int K)
+{
+    return ((N <= 8192 && K >= 2048) || K >= 8192) ? 4 : 2;
+}
+
 template <int NWAVE, int STAGES, int XJ, bool F32OUT, bool STAGEQ = false>
 int launch_skinny_cfg(const GemmArgs &g, hipStream_t st)
 {
@@ -1953,7 +1965,7 @@ inline bool stage_inside_launch_faster(int M, int N, int K, bool few_token_kerne
 // The instances of the kernel that quantizes the activations itself, by row count.
 inline int launch_skinny_staged_cfg(const GemmArgs &g, hipStream_t st)
 {
-    if (g.N < 2048) {   // few row blocks: K over four waves, as launch_skinny does for them
+    if (g.N < 2048 || skinny_waves_few_rows(g.N, g.K) == 4) {   // K over four waves, as launch_skinny does for these
         if (g.M <= 8)
             return launch_skinny_cfg<4, 2, 1, true, true>(g, st);
         if (g.M <= 16)
@@ -2256,7 +2268,7 @@ int launch_gemm(const GemmArgs &g_in, hipStream_t st)
     if (gemv_rows_applies(g.A, g.Bt, g.M, g.N, g.K) && gemv_rows_faster(g.M, g.N, g.K) && !config_set && !small_set)
         return launch_gemv_rows<false, F32OUT>(g, st);
     if (g.K % 256 == 0 && g.M <= 32 && g.N >= 2048 && !config_set)
-        return launch_skinny<F32OUT>(g, 2, st);  // weight streaming: enough row blocks to fill the chip
+        return launch_skinny<F32OUT>(g, skinny_waves_few_rows(g.N, g.K), st);  // weight streaming: enough row blocks to fill the chip
     if (g.K % 256 == 0 && !config_set && !small_set) {
         const int nwave = skinny_blocks_waves(g.M, g.N, g.K);
         if (nwave)
