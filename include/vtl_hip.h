@@ -259,12 +259,16 @@ const char *vtl_hip_last_error(void);
 const char *vtl_hip_version(void);
 /* Which tile configuration and how many K ranges the int8 tile kernels' cost
  * model picks for an M x N x K product (pure host arithmetic, no device
- * needed): config_index is what VTL_HIP_GEMM_CONFIG takes ("<index>,<splits>"),
- * tile_m x tile_n the block tile.  A test and tuning aid (tests/ checks the
- * choice against recorded timings); products that take one of the special
- * kernels (matrix-vector, weight streaming, small products) never ask it.
- * No counterpart in the reference. */
-int vtl_hip_gemm_tile_choice(int M, int N, int K, int *config_index, int *tile_m, int *tile_n, int *splits);
+ * needed), for vtl_hip_linear_i8_f32 / vtl_hip_gemm_i8_i32 (requant == 0) or
+ * for vtl_hip_linear_i8_requant (requant != 0: its second kernel runs whatever
+ * the split, so cutting K costs it less): config_index is what
+ * VTL_HIP_GEMM_CONFIG takes ("<index>,<splits>"), tile_m x tile_n the block
+ * tile.  A test and tuning aid (tests/ checks the choice against recorded
+ * timings); products that take one of the special kernels (matrix-vector,
+ * weight streaming, small products) never ask it.  No counterpart in the
+ * reference. */
+int vtl_hip_gemm_tile_choice(int M, int N, int K, int requant, int *config_index, int *tile_m, int *tile_n,
+                             int *splits);
 
 /* The library reads its tuning switches (environment variables VTL_HIP_*, used
  * by tests and tuning runs only) once, at the first call that looks at them;

@@ -31,7 +31,10 @@ from vtl_amd.tensor import HipTensor  # noqa: E402
 SHAPES = [(4096, 4096, 4096, "linear"), (128, 14336, 4096, "linear"), (256, 11008, 4096, "requant"),
           (256, 4096, 11008, "requant"), (6144, 6144, 2048, "linear"), (8192, 8192, 1024, "linear"),
           (1024, 4096, 4096, "linear"), (64, 14336, 4096, "linear"), (2048, 2048, 2048, "linear"),
-          (512, 8192, 8192, "linear")]
+          (512, 8192, 8192, "linear"),
+          # ragged M and long K, where constants fitted before the ragged-shape kernels were sped up
+          # chose a K split of the eight-wave tile at 25 to 50 % over the fastest entry
+          (96, 8192, 8192, "linear"), (129, 2048, 8192, "linear"), (400, 2048, 8192, "linear"), (128, 14336, 4096, "requant"), (512, 4096, 4096, "requant")]
 N_CONFIGS = 8
 SPLITS = (1, 2, 4, 8)
 

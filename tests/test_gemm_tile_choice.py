@@ -19,15 +19,16 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 SWEEP = json.load(open(os.path.join(HERE, "golden", "gemm_tile_sweep.json")))
 
 
-def _choice(m, n, k):
+def _choice(m, n, k, requant=False):
     idx, tm, tn, splits = C.c_int(), C.c_int(), C.c_int(), C.c_int()
-    capi.call("vtl_hip_gemm_tile_choice", m, n, k, C.byref(idx), C.byref(tm), C.byref(tn), C.byref(splits))
+    capi.call("vtl_hip_gemm_tile_choice", m, n, k, int(requant), C.byref(idx), C.byref(tm), C.byref(tn),
+              C.byref(splits))
     return idx.value, tm.value, tn.value, splits.value
 
 
 @pytest.mark.parametrize("rec", SWEEP["shapes"], ids=lambda r: f"{r['m']}x{r['n']}x{r['k']}")
 def test_choice_is_within_five_percent_of_the_fastest_measured(rec):
-    idx, tm, tn, splits = _choice(rec["m"], rec["n"], rec["k"])
+    idx, tm, tn, splits = _choice(rec["m"], rec["n"], rec["k"], rec["entry"] == "requant")
     key = f"{idx},{splits}"
     for regime in ("cached", "from_hbm"):
         times = rec[regime]
@@ -39,10 +40,10 @@ def test_choice_is_within_five_percent_of_the_fastest_measured(rec):
 def test_choice_reports_tile_shapes_and_rejects_bad_arguments():
     idx, tm, tn, splits = _choice(4096, 4096, 4096)
     assert (idx, tm, tn, splits) == (7, 256, 256, 1)           # the headline launch: one round of 256x256 tiles
-    idx, tm, tn, splits = _choice(256, 4096, 11008)
-    assert (tm, tn) == (128, 128) and splits == 4              # few tiles, long K: K is cut
+    idx, tm, tn, splits = _choice(256, 4096, 11008, requant=True)
+    assert (tm, tn) == (128, 64) and splits == 2               # few tiles, long K: K is cut
     one = C.c_int()
-    assert capi.status("vtl_hip_gemm_tile_choice", 0, 4, 4, C.byref(one), C.byref(one), C.byref(one),
+    assert capi.status("vtl_hip_gemm_tile_choice", 0, 4, 4, 0, C.byref(one), C.byref(one), C.byref(one),
                        C.byref(one)) == capi.ERR_INVALID_ARG
-    assert capi.status("vtl_hip_gemm_tile_choice", 4, 4, 4, None, C.byref(one), C.byref(one),
+    assert capi.status("vtl_hip_gemm_tile_choice", 4, 4, 4, 0, None, C.byref(one), C.byref(one),
                        C.byref(one)) == capi.ERR_INVALID_ARG

@@ -47,7 +47,8 @@ SIGNATURES = {
     "vtl_hip_gemm_i8_i32": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci]),
     "vtl_hip_linear_i8_f32": (_ci, [_vp, _vp, _ci, _vp, _vp, _ci, _vp, _vp, _ci, _ci, _ci, _ci]),
     "vtl_hip_linear_i8_requant": (_ci, [_vp, _vp, _ci, _vp, _vp, _ci, _vp, _ci, _vp, _vp, _vp, _ci, _ci, _ci]),
-    "vtl_hip_gemm_tile_choice": (_ci, [_ci, _ci, _ci, C.POINTER(_ci), C.POINTER(_ci), C.POINTER(_ci), C.POINTER(_ci)]),
+    "vtl_hip_gemm_tile_choice": (_ci, [_ci, _ci, _ci, _ci, C.POINTER(_ci), C.POINTER(_ci), C.POINTER(_ci),
+                                       C.POINTER(_ci)]),
     "vtl_hip_linear_f32_dynquant_workspace": (_sz, [_ci, _ci]),
     "vtl_hip_linear_f32_dynquant": (_ci, [_vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp, _sz]),
     "vtl_hip_linear_f32_dynquant_noalloc": (_ci, [_vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci]),

@@ -1820,13 +1820,13 @@ struct TileConfig {
     float busy_chip;    // factor on step_cycles when the whole chip runs such steps at once
 };
 constexpr TileConfig kTileConfigs[] = {
-    {32, 64, 357.f, 1, 1.2f}, {32, 128, 540.f, 2, 0.8f},
-    {64, 64, 410.f, 2, 1.03f},   // four stages
-    {64, 128, 594.f, 2, 0.88f},
-    {128, 64, 554.f, 1, 0.8f},  // four stages
-    {128, 128, 1050.f, 2, 0.84f},
-    {128, 128, 593.f, 1, 1.05f},  // four stages, eight waves: alone on its compute unit, for launches of one round
-    {256, 256, 2200.f, 1, 1.0f}};
+    {32, 64, 352.f, 1, 3.7f}, {32, 128, 483.f, 2, 1.07f},
+    {64, 64, 410.f, 2, 1.06f},   // four stages
+    {64, 128, 575.f, 2, 1.1f},
+    {128, 64, 518.f, 1, 1.2f},  // four stages
+    {128, 128, 1068.f, 2, 0.86f},
+    {128, 128, 636.f, 1, 1.45f},  // four stages, eight waves: alone on its compute unit, for launches of one round
+    {256, 256, 1996.f, 1, 0.83f}};
 constexpr int kNumTileConfigs = 8;
 
 // The epilogue addresses a tile's elements as a 32-bit offset (row in tile x N
@@ -1859,18 +1859,21 @@ int launch_config(int idx, const GemmArgs &g, int splits, hipStream_t st)
 // model, the larger of
 //   latency:    rounds of workgroups over the resident slots x K steps per workgroup x step cost
 //   throughput: all K steps of all workgroups x step cost x busy-chip factor / 256 compute units
-// plus, for split K, the extra launch and the pass over the partial sums.
-// The constants were fitted (random search, least mean log regret) to two
-// exhaustive timing sweeps of every tile and split count over 72 shapes - one
-// with the same weights every launch (up to 256 MB of them then stay in the
-// last-level cache), one with the weights taken from enough copies in turn that
-// every launch streams them from HBM, since which tile wins can depend on that
-// (160x14336x4096: 64x128 tiles take 20.5 us cached and 30.5 us from HBM,
-// 128x128 tiles 22.6 and 25.4) - the shapes of the decode and MLP-chain
-// workloads weighted six-fold, plus 15 shapes of 8192 / 10240 / 28672 / 57344
-// columns from HBM.  Mean regret 1.2 % cached and 0.7 % from HBM, worst 14 %
-// (192x8192x8192 cached, 512x8192x28672 from HBM).
-void choose_config(int M, int N, int K, int &best_idx, int &best_splits)
+// plus, for split K, the extra launch and the pass over the partial sums.  For the
+// requantizing linear, whose second kernel runs whatever the split, only the planes of
+// partial sums that kernel has to read count.
+// The constants were fitted (random search, least mean log regret) to exhaustive timing
+// sweeps of every tile and split count, each shape timed once with the same weights every
+// launch (up to 256 MB of them then stay in the last-level cache) and once with the weights
+// taken from enough copies in turn that every launch streams them from HBM, since which tile
+// wins can depend on that: 87 shapes from 40x11008x4096 to 8192^3, 153 with a ragged M
+// (33 ... 520 rows against nine weight matrices), and 90 through the requantizing entry
+// (48 ... 2048 rows), the shapes of the decode and MLP-chain workloads weighted six-fold.
+// Mean regret against the fastest measured entry 1.1 % cached and 1.2 % from HBM (worst 29 %:
+// 2048^3 through the requantizing entry, cached); the constants this replaces, fitted before
+// the kernels for ragged shapes were sped up, were at 5.4 % and 4.3 % on the same data, worst
+// 45 % and 53 % (config 6 with a K split chosen for 65 ... 400 rows and K >= 8192).
+void choose_config(int M, int N, int K, int &best_idx, int &best_splits, bool requant = false)
 {
     const int kt_all = (K + 127) / 128;
     float best = 3.0e38f;
@@ -1894,12 +1897,14 @@ void choose_config(int M, int N, int K, int &best_idx, int &best_splits)
                 break;
             const int64_t rounds = (tiles * s + 256 * c.wgs_per_cu - 1) / (256 * c.wgs_per_cu);
             const int steps = (kt_all + s - 1) / s;
-            const float fixed = c.bm == 256 ? 4000.f : 6000.f;   // fill and store of one workgroup
+            const float fixed = c.bm == 256 ? 4865.f : 6058.f;   // fill and store of one workgroup
             const float latency = (float)rounds * ((float)steps * c.step_cycles + fixed);
             const float throughput = (float)tiles * (float)s * (float)steps * c.step_cycles * c.busy_chip / 256.f + fixed;
             float cost = latency > throughput ? latency : throughput;
-            if (s > 1)
-                cost += 4500.f + (float)s * (float)M * (float)N * 4.0f / 1218.f;
+            if (requant)
+                cost += (float)s * (float)M * (float)N * 4.0f / 636.f;
+            else if (s > 1)
+                cost += 4084.f + (float)s * (float)M * (float)N * 4.0f / 606.f;
             if (cost < best) {
                 best = cost;
                 best_idx = i;
@@ -2191,7 +2196,9 @@ inline bool gemv_rows_faster(int M, int N, int K)
         return true;
     if (M <= 4)
         return K >= 2048 || N <= 8192;
-    return (int64_t)N * K <= (K >= 4096 ? (int64_t)24 << 20 : (int64_t)4 << 20);
+    // 5 to 8 rows: only small products (against four waves of the other kernel, which these
+    // shapes get: 8 x 4096 x 4096 5.5 against 4.8 us)
+    return (int64_t)N * K <= ((int64_t)4 << 20);
 }
 
 // Quantizing the rows inside every workgroup of the few-token kernel costs about 15 instructions
@@ -2365,7 +2372,7 @@ int vtl_hip_linear_i8_requant(const int8_t *A, const float *sa, int sa_per_row, 
         g.requant_codes = Yq;
         g.requant_scales = sy;
         int idx, splits;
-        choose_config(M, N, K, idx, splits);
+        choose_config(M, N, K, idx, splits, true);
         const Tuning &tn = tuning();
         if (tn.gemm_config >= 0 && tn.gemm_config < kNumTileConfigs) {   // VTL_HIP_GEMM_CONFIG, as in launch_gemm
             idx = tn.gemm_config;
@@ -2387,12 +2394,13 @@ int vtl_hip_linear_i8_requant(const int8_t *A, const float *sa, int sa_per_row, 
     return launch_quantize_rows(Y, M, N, Yq, sy, current_stream());
 }
 
-int vtl_hip_gemm_tile_choice(int M, int N, int K, int *config_index, int *tile_m, int *tile_n, int *splits)
+int vtl_hip_gemm_tile_choice(int M, int N, int K, int requant, int *config_index, int *tile_m, int *tile_n,
+                             int *splits)
 {
     if (!config_index || !tile_m || !tile_n || !splits || M <= 0 || N <= 0 || K <= 0)
         return VTL_HIP_ERR_INVALID_ARG;
     int idx, s;
-    choose_config(M, N, K, idx, s);
+    choose_config(M, N, K, idx, s, requant != 0);
     if (idx < 0)
         return VTL_HIP_ERR_UNSUPPORTED;
     *config_index = idx;
