@@ -101,6 +101,11 @@ int vtl_hip_event_elapsed_ms(void *start, void *stop, float *ms);
 
 /* absmax_out[0] = max |x| over the tensor (per_row == 0) or absmax_out[r] =
  * max |x[r, :]| (per_row != 0).  NaN elements are ignored; empty -> 0.
+ * The whole-tensor maximum is collected in a few bytes of device memory that the
+ * library keeps per stream (for the first 16 streams of a device that make such
+ * a call; calls on further streams, and calls recorded into a graph, clear and
+ * use absmax_out itself, one launch more).  Calls on one stream are ordered;
+ * calls on different streams do not disturb each other.
  * Replaces Tensor.abs (math.v:11-16) + max_axis (reduction.v:163-232) /
  * stats.max (stats/stats.v:401-407). */
 int vtl_hip_absmax_f32(const float *x, int64_t rows, int64_t cols, int per_row,
@@ -108,7 +113,11 @@ int vtl_hip_absmax_f32(const float *x, int64_t rows, int64_t cols, int per_row,
 
 /* scale = absmax / 127 (f32 division); q = clamp(round_half_even(x / scale),
  * -127, 127) with NaN -> 0 and scale 0 -> all codes 0.  scale_out receives 1
- * (per_row == 0) or `rows` scales.  Replaces divide_scalar (math_op.v:103-111)
+ * (per_row == 0) or `rows` scales.  per_row != 0 is one launch; per_row == 0 is
+ * one launch up to 65536 elements, two up to 2^24 (absmax as in
+ * vtl_hip_absmax_f32, then a pass that derives the scale from it), four beyond
+ * or where vtl_hip_absmax_f32 has no memory of its own for the stream.
+ * Replaces divide_scalar (math_op.v:103-111)
  * + round_to_even (math.v:570-574) + clamp (autograd/variable_ops.v:228-248)
  * + as_i8 (cast.v:107-121). */
 int vtl_hip_quantize_f32_i8(const float *x, int64_t rows, int64_t cols, int per_row,

@@ -206,6 +206,144 @@ def test_engineered_near_ties_per_row(hip):
     assert np.array_equal(s.cpu(), sr) and np.array_equal(q.cpu(), qr)
 
 
+def _tensor_quantize(X, rows, cols, Q, S):
+    capi.call("vtl_hip_quantize_f32_i8", X.ptr, rows, cols, 0, Q.ptr, S.ptr)
+
+
+@pytest.mark.parametrize("shape", [(1, 65540), (257, 257), (1000, 1001), (1024, 1024), (2048, 4100), (4096, 4096),
+                                   (4096, 4097)])
+def test_whole_tensor_quantize_in_two_launches_equals_four(hip, shape, knobs):
+    """Above 65536 elements a whole-tensor quantize collects the absmax in cells that the library
+    keeps per stream and its second launch derives the scale from them (up to 16 M elements;
+    the last shape is past that).  Codes and scale must be those of the four-launch form and
+    of the oracle, call after call: a call must not see the maximum of the one before."""
+    rows, cols = shape
+    rng = np.random.Generator(np.random.Philox(rows * 31 + cols))
+    base = rng.standard_normal(shape, dtype=np.float32)
+    base.reshape(-1)[:4] = [0.5, 1.5, -2.5, 3.5]
+    X = raw_device_buffer(base.nbytes + 16)
+    Q = raw_device_buffer(base.size + 16)
+    S, A = raw_device_buffer(64), raw_device_buffer(64)
+    small = rows * cols <= 1 << 21
+    # descending magnitudes: a maximum left over from an earlier call would show
+    for step, (mag, off) in enumerate(((64.0, 0), (1.0, 0), (1.0, 4), (0.015625, 0), (0.0, 0))):
+        if off and not small:
+            continue
+        x = base * np.float32(mag)
+        if step == 1:
+            x[rows // 2, cols // 3] = np.nan        # ignored by the absmax, code 0
+        h2d(X.ptr + off, x)
+        want_q, want_s = oracle.quantize(x, False, threads=CPU_THREADS)
+        got = {}
+        for form in ("two", "four"):
+            if form == "four":
+                knobs.setenv("VTL_HIP_QUANT_FOUR_LAUNCHES", "1")
+            capi.call("vtl_hip_memset", S.ptr, 0xFF, 64)
+            capi.call("vtl_hip_quantize_f32_i8", X.ptr + off, rows, cols, 0, Q.ptr + off // 4, S.ptr)
+            capi.call("vtl_hip_absmax_f32", X.ptr + off, rows, cols, 0, A.ptr)
+            got[form] = (d2h(Q.ptr + off // 4, shape, np.int8), d2h(S.ptr, 1, np.float32), d2h(A.ptr, 1, np.float32))
+            if form == "four":
+                knobs.delenv("VTL_HIP_QUANT_FOUR_LAUNCHES")
+        for form, (codes, scale, amax) in got.items():
+            assert scale.view(np.uint32)[0] == want_s.view(np.uint32).reshape(-1)[0], (form, step)
+            assert amax[0] == oracle.absmax(x, False).reshape(-1)[0], (form, step)
+            assert np.array_equal(codes, want_q), (form, step)
+    for h in (X, Q, S, A):
+        h.release()
+
+
+def test_whole_tensor_quantize_on_many_streams(hip):
+    """Every stream has absmax cells of its own (the first 16 streams that ask; further ones
+    take the four-launch form): calls enqueued on 20 streams without waiting in between, three
+    rounds with a different tensor per stream and round, each give their own scale and codes."""
+    import ctypes as C
+    hiprt = C.CDLL("libamdhip64.so")
+    rows, cols = 300, 1000
+    rng = np.random.Generator(np.random.Philox(4242))
+    lanes = []
+    try:
+        for i in range(20):
+            st = C.c_void_p()
+            assert hiprt.hipStreamCreate(C.byref(st)) == 0
+            xs = [rng.standard_normal((rows, cols), dtype=np.float32) * np.float32(2.0 ** (i % 7 - rnd)) for rnd in range(3)]
+            lanes.append({"stream": st, "xs": xs, "X": [dev(x) for x in xs],
+                          "Q": [raw_device_buffer(rows * cols) for _ in xs], "S": [raw_device_buffer(64) for _ in xs]})
+        for rnd in range(3):
+            for ln in lanes:
+                capi.call("vtl_hip_set_stream", ln["stream"])
+                _tensor_quantize(ln["X"][rnd], rows, cols, ln["Q"][rnd], ln["S"][rnd])
+        for ln in lanes:
+            capi.call("vtl_hip_set_stream", ln["stream"])
+            capi.call("vtl_hip_sync")
+        for i, ln in enumerate(lanes):
+            for rnd in range(3):
+                want_q, want_s = oracle.quantize(ln["xs"][rnd], False, threads=CPU_THREADS)
+                assert d2h(ln["S"][rnd].ptr, 1, np.float32)[0] == want_s.reshape(-1)[0], (i, rnd)
+                assert np.array_equal(d2h(ln["Q"][rnd].ptr, (rows, cols), np.int8), want_q), (i, rnd)
+    finally:
+        capi.call("vtl_hip_set_stream", None)
+        capi.call("vtl_hip_sync")
+        for ln in lanes:
+            hiprt.hipStreamDestroy(ln["stream"])
+            for t in [*ln["X"], *ln["Q"], *ln["S"]]:
+                t.release()
+
+
+def test_whole_tensor_quantize_under_stream_capture(hip):
+    """The cells a call uses alternate from call to call, which a recorded graph cannot follow:
+    under capture the library records the form that uses the caller's memory only, and replays
+    with eager calls between them all give the oracle's bits."""
+    import ctypes as C
+    hiprt = C.CDLL("libamdhip64.so")
+    stream, graph, gexec = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    assert hiprt.hipStreamCreate(C.byref(stream)) == 0
+    rows, cols = 512, 1024
+    rng = np.random.Generator(np.random.Philox(515))
+    x = rng.standard_normal((rows, cols), dtype=np.float32)
+    X = dev(x)
+    Q, S, A = raw_device_buffer(rows * cols), raw_device_buffer(64), raw_device_buffer(64)
+
+    def call():
+        _tensor_quantize(X, rows, cols, Q, S)
+        capi.call("vtl_hip_absmax_f32", X.ptr, rows, cols, 0, A.ptr)
+
+    def check(xr, what):
+        want_q, want_s = oracle.quantize(xr, False, threads=CPU_THREADS)
+        assert d2h(S.ptr, 1, np.float32)[0] == want_s.reshape(-1)[0], what
+        assert d2h(A.ptr, 1, np.float32)[0] == np.abs(xr).max(), what
+        assert np.array_equal(d2h(Q.ptr, (rows, cols), np.int8), want_q), what
+
+    try:
+        capi.call("vtl_hip_set_stream", stream)
+        call()
+        capi.call("vtl_hip_sync")
+        check(x, "eager")
+        assert hiprt.hipStreamBeginCapture(stream, 0) == 0
+        call()
+        assert hiprt.hipStreamEndCapture(stream, C.byref(graph)) == 0
+        assert hiprt.hipGraphInstantiate(C.byref(gexec), graph, None, None, C.c_size_t(0)) == 0
+        for rep in range(4):
+            xr = (rng.standard_normal((rows, cols)) * 2.0 ** (3 - rep)).astype(np.float32)
+            capi.call("vtl_hip_memcpy_h2d", X.ptr, xr.ctypes.data, xr.nbytes)
+            if rep % 2:
+                call()
+                capi.call("vtl_hip_sync")
+                check(xr, f"eager {rep}")
+                capi.call("vtl_hip_memset", Q.ptr, 0, rows * cols)
+            assert hiprt.hipGraphLaunch(gexec, stream) == 0
+            capi.call("vtl_hip_sync")
+            check(xr, f"replay {rep}")
+    finally:
+        capi.call("vtl_hip_set_stream", None)
+        if gexec:
+            hiprt.hipGraphExecDestroy(gexec)
+        if graph:
+            hiprt.hipGraphDestroy(graph)
+        hiprt.hipStreamDestroy(stream)
+        for t in (X, Q, S, A):
+            t.release()
+
+
 def test_relu_matches_oracle(hip):
     x = np.array([-1.0, -0.0, 0.0, 2.5, -1e-30, np.inf, -np.inf, np.nan] * 37, np.float32)
     t = dev(x)

@@ -38,6 +38,15 @@ void *library_workspace(size_t bytes, int slot = 0);
 // not fit the static scratch or would have to allocate during a stream capture).
 int workspace_status();
 
+// A small index (0 .. kStreamSlots - 1) that belongs to `st` on the current device, for code
+// that keeps a little state in device memory between its launches and must not share it with
+// work that may run at the same time: the first kStreamSlots streams that ask get one each, for
+// as long as the process lives (a stream handle that is reused inherits its predecessor's
+// index, which is as good).  -1 when none is left, when the stream is being captured into a
+// graph (a replay would meet the state of another moment) or when that cannot be found out.
+constexpr int kStreamSlots = 16;
+int stream_slot(hipStream_t st);
+
 // Static per-device scratch for the entry point that allocates nothing, and the
 // scope during which library_workspace() serves from it.  static_scratch()
 // returns the device address of the current device's array (nullptr on error).
@@ -63,6 +72,7 @@ struct Tuning {
     int gemm_splits = 1;
     bool no_fused_requant = false;  // VTL_HIP_NO_FUSED_REQUANT: linear, then the row quantizer
     int requant_wide = 0;           // VTL_HIP_REQUANT_WIDE: 1 row maxima in the tile kernel + wide quantizer, 0 one workgroup per row
+    bool quant_four_launches = false;  // VTL_HIP_QUANT_FOUR_LAUNCHES: whole-tensor quantize as clear + absmax + scale + quantize (tests)
     bool no_fused_decode = false;   // VTL_HIP_NO_FUSED_DECODE: quantizer launch in front of the linear
     int stage_spin = 4096;          // VTL_HIP_STAGE_SPIN: polls a workgroup of the decode launch waits for the quantized rows (0: none, tests)
     int skinny_tiled = -1;          // VTL_HIP_SKINNY_TILED: 1 / 0 force the 32x32-block weight-streaming kernel for M > 32

@@ -848,7 +848,7 @@ __device__ __forceinline__ void lds_barrier()
 // spin_limit polls a workgroup quantizes all M rows itself (the same values into the same
 // places) and goes on, so the launch drains whatever the order in which workgroups start.
 // Launches that share a slot must not overlap.
-constexpr int kStageSlots = 16;
+constexpr int kStageSlots = vtlhip::kStreamSlots;
 constexpr int kStageCopies = 64;
 constexpr int kStageMaxK = 8192;
 __device__ unsigned g_stage_count[kStageSlots * kStageCopies * 64];
@@ -1987,38 +1987,14 @@ inline int launch_skinny_staged_cfg(const GemmArgs &g, hipStream_t st)
 // Host side of the launch that quantizes the activations itself.  Its workgroups meet on a
 // counter that only grows, so the host has to know what every earlier launch added to it and
 // launches that share a counter must run one after the other: each stream gets a counter of
-// its own (the first kStageSlots streams that ask, per device, for as long as the process
-// lives; a stream handle that is reused inherits its predecessor's counter, which is as good),
-// and the value it will reach is kept beside it.  No counter is handed out while the stream is
-// being captured (a replay would wait for a value that was reached long ago), nor when the
-// capture state cannot be queried.
+// its own (the index vtlhip::stream_slot gives it: one of the first kStageSlots streams per
+// device that ask), and the value it will reach is kept beside it.  No counter is handed out
+// while the stream is being captured (a replay would wait for a value that was reached long
+// ago), nor when the capture state cannot be queried.
 struct StageCounters {
     std::mutex lock;
-    hipStream_t stream[kStageSlots] = {};
-    bool taken[kStageSlots] = {};
     unsigned counted[kStageSlots] = {};
 };
-
-inline int stage_counter_of(StageCounters &c, hipStream_t st)
-{
-    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(st, &capturing) != hipSuccess) {
-        (void)hipGetLastError();
-        return -1;
-    }
-    if (capturing != hipStreamCaptureStatusNone)
-        return -1;
-    for (int i = 0; i < kStageSlots; i++)
-        if (c.taken[i] && c.stream[i] == st)
-            return i;
-    for (int i = 0; i < kStageSlots; i++)
-        if (!c.taken[i]) {
-            c.taken[i] = true;
-            c.stream[i] = st;
-            return i;
-        }
-    return -1;
-}
 
 // The weight-streaming launch that quantizes the f32 activations g.xf32 itself, into
 // g.stage_codes / g.stage_scales (which g.A / g.sa name too).  M <= 32, K <= kStageMaxK.
@@ -2029,7 +2005,7 @@ inline int launch_skinny_staged(GemmArgs g, hipStream_t st, bool &launched)
     static PerDevice<StageCounters> counters;
     StageCounters &c = counters.get();
     std::lock_guard<std::mutex> hold(c.lock);
-    const int slot = stage_counter_of(c, st);
+    const int slot = vtlhip::stream_slot(st);
     launched = slot >= 0;
     if (!launched)
         return VTL_HIP_OK;

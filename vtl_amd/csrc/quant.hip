@@ -12,6 +12,9 @@
 // The division is the correctly rounded one.  The quotient is first estimated
 // with x * (1/scale); only when that estimate is too close to a rounding tie
 // to decide the integer is the exact division evaluated (see quant_code).
+#include <atomic>
+#include <mutex>
+
 #include "common.hpp"
 #include "quant_device.hpp"
 
@@ -31,6 +34,20 @@ __device__ __forceinline__ int row_head(int64_t start, int64_t cols)
 }
 
 // ---- absmax ----------------------------------------------------------------
+
+// A whole-tensor maximum is collected by atomic maxima of the workgroups.  On one address those
+// queue up (6 to 7 ns each: 4096 x 4096 took 28 us with 2048 workgroups, against 8.8 us for the
+// per-row kernel over the same bytes), so a set of kAbsmaxCells cells 128 bytes apart takes
+// them, workgroup b using cell b % kAbsmaxCells, and whoever wants the maximum reads them all.
+constexpr int kAbsmaxCells = 64;
+constexpr int kCellStride = 32;   // in 4-byte units
+
+// The maximum over a set of cells; every lane of the calling wave gets it.
+__device__ __forceinline__ float absmax_of_cells(const unsigned *cells)
+{
+    return wave_max(__uint_as_float(cells[(threadIdx.x & (kAbsmaxCells - 1)) * kCellStride]));
+}
+
 
 // One workgroup per row, strided loop over the row.
 template <int T, int VEC>
@@ -72,9 +89,12 @@ __global__ __launch_bounds__(T) void absmax_rows_kernel(const float *__restrict_
 
 // Whole-tensor absmax: grid-stride pass, one atomic max per workgroup on the
 // bit pattern (non-negative floats order like unsigned integers).
-template <int T>
+// KEEP: ordinary loads, for a tensor that a second pass reads again while the last-level cache
+// still holds it; otherwise non-temporal ones.
+template <int T, bool KEEP = false>
 __global__ __launch_bounds__(T) void absmax_flat_kernel(const float *__restrict__ x, int64_t n,
-                                                        int vec_ok, unsigned *__restrict__ out_bits)
+                                                        int vec_ok, unsigned *__restrict__ out_bits,
+                                                        int cells)
 {
     __shared__ float smem[T / 64];
     float m = 0.0f;
@@ -85,10 +105,18 @@ __global__ __launch_bounds__(T) void absmax_flat_kernel(const float *__restrict_
         const int64_t nv = n >> 2;
         int64_t i = tid;
         for (; i + 3 * stride < nv; i += 4 * stride) {
-            const float4_t v0 = __builtin_nontemporal_load(xv + i);
-            const float4_t v1 = __builtin_nontemporal_load(xv + i + stride);
-            const float4_t v2 = __builtin_nontemporal_load(xv + i + 2 * stride);
-            const float4_t v3 = __builtin_nontemporal_load(xv + i + 3 * stride);
+            float4_t v0, v1, v2, v3;
+            if constexpr (KEEP) {
+                v0 = xv[i];
+                v1 = xv[i + stride];
+                v2 = xv[i + 2 * stride];
+                v3 = xv[i + 3 * stride];
+            } else {
+                v0 = __builtin_nontemporal_load(xv + i);
+                v1 = __builtin_nontemporal_load(xv + i + stride);
+                v2 = __builtin_nontemporal_load(xv + i + 2 * stride);
+                v3 = __builtin_nontemporal_load(xv + i + 3 * stride);
+            }
             m = absmax4(absmax4(absmax4(absmax4(m, v0), v1), v2), v3);
         }
         for (; i < nv; i += stride)
@@ -101,7 +129,7 @@ __global__ __launch_bounds__(T) void absmax_flat_kernel(const float *__restrict_
     }
     m = block_max<T>(m, smem);
     if (threadIdx.x == 0)
-        atomicMax(out_bits, __float_as_uint(m));
+        atomicMax(out_bits + (blockIdx.x % (unsigned)cells) * kCellStride, __float_as_uint(m));
 }
 
 __global__ void fill_u32_kernel(unsigned *p, unsigned v, int64_t n)
@@ -116,6 +144,15 @@ __global__ void scale_from_absmax_kernel(float *inout, int64_t n)
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n)
         inout[i] = inout[i] / 127.0f;
+}
+
+// One wave: the maximum over a set of cells to *out, and the cells back to zero.
+__global__ __launch_bounds__(64) void absmax_cells_reduce_kernel(unsigned *cells, float *out)
+{
+    const float m = absmax_of_cells(cells);
+    cells[threadIdx.x * kCellStride] = 0u;
+    if (threadIdx.x == 0)
+        *out = m;
 }
 
 // ---- fused per-row absmax + quantize ---------------------------------------
@@ -225,18 +262,35 @@ __global__ __launch_bounds__(T) void quantize_rows_loop_kernel(const float *__re
 // (VEC == 1).  The grid is one-dimensional and chunk-major (block = row *
 // chunks_per_row + chunk), so that workgroups dispatched back to back touch
 // adjacent memory; per_row == 0 treats the tensor as one row of `cols` elements.
-template <int T, int NV, int VEC>
+// FROM_ABSMAX (whole tensor only): `scale` points at a set of cells as absmax_flat_kernel
+// leaves them; every workgroup derives the scale from their maximum, the first also stores the
+// scale to scale_out and clears the set clear_cells (the one the next such call on this stream
+// will collect its absmax in).
+template <int T, int NV, int VEC, bool FROM_ABSMAX = false>
 __global__ __launch_bounds__(T) void quantize_scaled_kernel(const float *__restrict__ x,
                                                             const float *__restrict__ scale,
                                                             int per_row, int64_t cols,
                                                             unsigned chunks_per_row,
-                                                            int8_t *__restrict__ q)
+                                                            int8_t *__restrict__ q,
+                                                            float *__restrict__ scale_out = nullptr,
+                                                            unsigned *__restrict__ clear_cells = nullptr)
 {
     const int64_t row = per_row ? (int64_t)(blockIdx.x / chunks_per_row) : 0;
     const int64_t chunk = per_row ? (int64_t)(blockIdx.x % chunks_per_row) : (int64_t)blockIdx.x;
     const float *xr = x + row * cols;
     int8_t *qr = q + row * cols;
-    const QuantScale p = make_quant_scale(scale[row]);
+    float row_scale;
+    if constexpr (FROM_ABSMAX) {
+        row_scale = absmax_of_cells(reinterpret_cast<const unsigned *>(scale)) / 127.0f;
+        if (blockIdx.x == 0 && threadIdx.x < kAbsmaxCells) {
+            clear_cells[threadIdx.x * kCellStride] = 0u;
+            if (threadIdx.x == 0)
+                *scale_out = row_scale;
+        }
+    } else {
+        row_scale = scale[row];
+    }
+    const QuantScale p = make_quant_scale(row_scale);
     if constexpr (VEC == 4) {
         const float4_t *xv = reinterpret_cast<const float4_t *>(xr);
         unsigned *qv = reinterpret_cast<unsigned *>(qr);
@@ -481,6 +535,96 @@ int check_2d(const void *a, const void *b, int64_t rows, int64_t cols)
     return VTL_HIP_OK;
 }
 
+// Whole-tensor quantization in two launches.  The absmax pass needs cells that hold zero when
+// it starts and the quantize pass must find the maximum in them: a cell in the caller's
+// scale_out would have to be cleared by a launch of its own and turned into the scale by
+// another.  Instead every stream index (vtlhip::stream_slot) owns two sets of cells in device
+// memory that the library uses in turn: a call collects its maximum in one, and its quantize
+// pass clears the other for the next call on that stream, whose launches come later in stream
+// order.  (vtl_hip_absmax_f32 uses the set whose turn it is and clears it itself.)  All cells
+// start as zero.  A call whose launches fail leaves the sets in an unknown state: the index
+// then goes back to the forms that use the caller's memory only, for good.
+constexpr int kCellSet = kAbsmaxCells * kCellStride;
+__device__ unsigned g_absmax_cells[vtlhip::kStreamSlots * 2 * kCellSet];
+
+struct AbsmaxCells {
+    std::mutex lock;
+    std::atomic<unsigned *> base{nullptr};   // device address of this device's g_absmax_cells
+    unsigned char turn[vtlhip::kStreamSlots] = {};
+    bool unusable[vtlhip::kStreamSlots] = {};
+};
+
+AbsmaxCells *absmax_cells_of_device()
+{
+    static AbsmaxCells cells[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    AbsmaxCells &c = cells[dev];
+    if (!c.base.load(std::memory_order_acquire)) {
+        void *ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_absmax_cells)) != hipSuccess) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        c.base.store(static_cast<unsigned *>(ptr), std::memory_order_release);
+    }
+    return &c;
+}
+
+// max |x| over n > 0 elements into a set of kAbsmaxCells cells that hold zero (the bits of a
+// non-negative float).
+int launch_absmax_cells(const float *x, int64_t n, unsigned *cells, bool keep_cached, hipStream_t s)
+{
+    // Up to 8 M elements: workgroups of 256 threads with 128 bytes per thread (1024 x 4096: 7.5
+    // against 8.8 us for the form below).  Beyond: at most two workgroups of 1024 threads per
+    // compute unit, which stream better (16384 x 16384: 372 against 424 us).
+    const int vec_ok = aligned(x, 16) ? 1 : 0;
+    const int64_t small = (n / 4 + 256 * 8 - 1) / (256 * 8);
+    if (small <= 1024) {
+        const dim3 grid((unsigned)(small < 1 ? 1 : small));
+        if (keep_cached)
+            hipLaunchKernelGGL((absmax_flat_kernel<256, true>), grid, dim3(256), 0, s, x, n, vec_ok, cells,
+                               kAbsmaxCells);
+        else
+            hipLaunchKernelGGL((absmax_flat_kernel<256, false>), grid, dim3(256), 0, s, x, n, vec_ok, cells,
+                               kAbsmaxCells);
+    } else {
+        int64_t blocks = (n / 4 + 1024 * 4 - 1) / (1024 * 4);
+        if (blocks > 512)
+            blocks = 512;
+        if (keep_cached)
+            hipLaunchKernelGGL((absmax_flat_kernel<1024, true>), dim3((unsigned)blocks), dim3(1024), 0, s, x, n,
+                               vec_ok, cells, kAbsmaxCells);
+        else
+            hipLaunchKernelGGL((absmax_flat_kernel<1024, false>), dim3((unsigned)blocks), dim3(1024), 0, s, x, n,
+                               vec_ok, cells, kAbsmaxCells);
+    }
+    return check_launch("absmax_flat_kernel");
+}
+
+// The same into the single cell *cell (caller's memory, cleared before).
+int launch_absmax_flat(const float *x, int64_t n, unsigned *cell, hipStream_t s)
+{
+    // One address for every workgroup's atomic maximum: few, large workgroups (at most two of
+    // 1024 threads per compute unit), small ones only while there are at most 512 of them.
+    const int vec_ok = aligned(x, 16) ? 1 : 0;
+    const int64_t small = (n / 4 + 256 * 4 - 1) / (256 * 4);
+    if (small <= 512) {
+        hipLaunchKernelGGL((absmax_flat_kernel<256, false>), dim3((unsigned)(small < 1 ? 1 : small)), dim3(256), 0, s,
+                           x, n, vec_ok, cell, 1);
+    } else {
+        int64_t blocks = (n / 4 + 1024 * 4 - 1) / (1024 * 4);
+        if (blocks > 512)
+            blocks = 512;
+        hipLaunchKernelGGL((absmax_flat_kernel<1024, false>), dim3((unsigned)blocks), dim3(1024), 0, s, x, n, vec_ok,
+                           cell, 1);
+    }
+    return check_launch("absmax_flat_kernel");
+}
+
 int launch_fill_zero(float *p, int64_t n, hipStream_t st)
 {
     const int64_t blocks = (n + 255) / 256;
@@ -595,21 +739,33 @@ int vtl_hip_absmax_f32(const float *x, int64_t rows, int64_t cols, int per_row, 
                                cols, absmax_out);
         return check_launch("absmax_rows_kernel");
     }
+    const int64_t n = rows * cols;
+    if (n > 0) {
+        // into the stream's cells, then one wave takes their maximum to absmax_out and clears them
+        const int slot = tuning().quant_four_launches ? -1 : vtlhip::stream_slot(s);
+        AbsmaxCells *cells = slot >= 0 ? absmax_cells_of_device() : nullptr;
+        if (cells) {
+            std::lock_guard<std::mutex> hold(cells->lock);
+            if (!cells->unusable[slot]) {
+                unsigned *mine = cells->base.load(std::memory_order_acquire) +
+                                 (slot * 2 + cells->turn[slot]) * kCellSet;
+                st = launch_absmax_cells(x, n, mine, false, s);
+                if (st == VTL_HIP_OK) {
+                    hipLaunchKernelGGL(absmax_cells_reduce_kernel, dim3(1), dim3(64), 0, s, mine, absmax_out);
+                    st = check_launch("absmax_cells_reduce_kernel");
+                }
+                if (st != VTL_HIP_OK)
+                    cells->unusable[slot] = true;
+                return st;
+            }
+        }
+    }
     st = launch_fill_zero(absmax_out, 1, s);
     if (st != VTL_HIP_OK)
         return st;
-    const int64_t n = rows * cols;
     if (n == 0)
         return VTL_HIP_OK;
-    const int vec_ok = aligned(x, 16) ? 1 : 0;
-    int64_t blocks = (n / 4 + 256 * 8 - 1) / (256 * 8);
-    if (blocks < 1)
-        blocks = 1;
-    if (blocks > 256 * 16)
-        blocks = 256 * 16;
-    hipLaunchKernelGGL((absmax_flat_kernel<256>), dim3((unsigned)blocks), dim3(256), 0, s, x, n, vec_ok,
-                       reinterpret_cast<unsigned *>(absmax_out));
-    return check_launch("absmax_flat_kernel");
+    return launch_absmax_flat(x, n, reinterpret_cast<unsigned *>(absmax_out), s);
 }
 
 int vtl_hip_quantize_with_scale_f32_i8(const float *x, const float *scale, int64_t rows,
@@ -667,6 +823,46 @@ int vtl_hip_quantize_f32_i8(const float *x, int64_t rows, int64_t cols, int per_
     const int64_t total = rows * cols;
     if (total > 0 && total <= 4 * 1024 * 16 && total % 4 == 0 && aligned(x, 16) && aligned(q, 4))
         return launch_quantize_rows(x, 1, total, q, scale_out, s);
+    if (total > 0 && total <= ((int64_t)1 << 24)) {
+        // whole tensor in two launches: absmax into one of the stream's two sets of cells, then
+        // the quantize pass, whose workgroups derive the scale from them (1024 x 1024: 6.0
+        // against 10.8 us for the four launches below, 4096 x 4096: 24.6 against 32.6 us).  Up
+        // to 16 M elements: beyond, reading the cells in every workgroup costs more than the two
+        // launches (8192 x 8192: 106 against 98 us).
+        const int slot = tuning().quant_four_launches ? -1 : vtlhip::stream_slot(s);
+        AbsmaxCells *cells = slot >= 0 ? absmax_cells_of_device() : nullptr;
+        constexpr int T = 512, NV = 2;
+        const bool vec = aligned(x, 16) && aligned(q, 4);
+        const int64_t per_chunk = vec ? 4 * T * NV : T * NV;
+        const int64_t chunks = (total + per_chunk - 1) / per_chunk;
+        if (cells && chunks <= kMaxGridX) {
+            std::lock_guard<std::mutex> hold(cells->lock);
+            if (!cells->unusable[slot]) {
+                unsigned *pair = cells->base.load(std::memory_order_acquire) + slot * 2 * kCellSet;
+                unsigned *mine = pair + cells->turn[slot] * kCellSet;
+                unsigned *next = pair + (cells->turn[slot] ^ 1) * kCellSet;
+                // (ordinary loads: the second pass finds the tensor in the last-level cache)
+                st = launch_absmax_cells(x, total, mine, true, s);
+                if (st == VTL_HIP_OK) {
+                    const dim3 grid((unsigned)chunks);
+                    if (vec)
+                        hipLaunchKernelGGL((quantize_scaled_kernel<T, NV, 4, true>), grid, dim3(T), 0, s, x,
+                                           reinterpret_cast<const float *>(mine), 0, total, (unsigned)chunks, q,
+                                           scale_out, next);
+                    else
+                        hipLaunchKernelGGL((quantize_scaled_kernel<T, NV, 1, true>), grid, dim3(T), 0, s, x,
+                                           reinterpret_cast<const float *>(mine), 0, total, (unsigned)chunks, q,
+                                           scale_out, next);
+                    st = check_launch("quantize_scaled_kernel");
+                }
+                if (st == VTL_HIP_OK)
+                    cells->turn[slot] ^= 1;
+                else
+                    cells->unusable[slot] = true;
+                return st;
+            }
+        }
+    }
     // whole tensor: absmax pass, scale in place, then the scaled quantize pass
     st = vtl_hip_absmax_f32(x, rows, cols, 0, scale_out);
     if (st != VTL_HIP_OK)

@@ -69,6 +69,7 @@ static const Tuning *read_tuning(bool force)
     }
     t->no_fused_requant = flag("VTL_HIP_NO_FUSED_REQUANT");
     t->requant_wide = number("VTL_HIP_REQUANT_WIDE", 0);
+    t->quant_four_launches = flag("VTL_HIP_QUANT_FOUR_LAUNCHES");
     t->no_fused_decode = flag("VTL_HIP_NO_FUSED_DECODE");
     t->stage_spin = number("VTL_HIP_STAGE_SPIN", 4096);
     if (t->stage_spin < 0 || t->stage_spin > (1 << 20))
@@ -106,6 +107,38 @@ static int current_device()
         return -1;
     }
     return dev;
+}
+
+int stream_slot(hipStream_t st)
+{
+    struct Table {
+        std::mutex lock;
+        hipStream_t stream[kStreamSlots] = {};
+        bool taken[kStreamSlots] = {};
+    };
+    static Table tables[kMaxDevices];
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &capturing) != hipSuccess) {
+        (void)hipGetLastError();
+        return -1;
+    }
+    if (capturing != hipStreamCaptureStatusNone)
+        return -1;
+    const int dev = current_device();
+    if (dev < 0)
+        return -1;
+    Table &t = tables[dev];
+    std::lock_guard<std::mutex> hold(t.lock);
+    for (int i = 0; i < kStreamSlots; i++)
+        if (t.taken[i] && t.stream[i] == st)
+            return i;
+    for (int i = 0; i < kStreamSlots; i++)
+        if (!t.taken[i]) {
+            t.taken[i] = true;
+            t.stream[i] = st;
+            return i;
+        }
+    return -1;
 }
 
 void *static_scratch()
