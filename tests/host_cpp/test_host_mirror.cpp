@@ -197,6 +197,13 @@ int main(int argc, char **argv)
         auto chain = s.mlp_forward_i8(x, M, {&w, &w2}, {&b, &b2}, {K, N, O}, {true, false});
         auto h_relu = ref_linear(x, M, K, w, N, b, true);
         CHECK(chain == ref_linear(h_relu, M, N, w2, O, b2, false));
+        // a few tokens take the route on which every layer quantizes its own input: same bits
+        for (int few : {1, 5, 32}) {
+            std::vector<float> xf(x.begin(), x.begin() + (size_t)few * K);
+            auto got = s.mlp_forward_i8(xf, few, {&w, &w2}, {&b, &b2}, {K, N, O}, {true, false});
+            auto hf = ref_linear(xf, few, K, w, N, b, true);
+            CHECK(got == ref_linear(hf, few, N, w2, O, b2, false));
+        }
         s.release();
     }
     // la.matmul and LinearGate.backward with f64 accumulation vs oracle: integer-valued

@@ -127,6 +127,27 @@ def test_mlp_chain_config(hip):
     model.release()
 
 
+@pytest.mark.parametrize("m", [1, 8, 32, 33])
+def test_mlp_chain_with_few_tokens(hip, m):
+    """Up to 32 tokens Sequential keeps the activations f32 between the layers and every layer
+    quantizes its input inside its own launch; from 33 on codes go from layer to layer.  Both
+    give the oracle's bits (4096 -> 2048 -> ReLU -> 1024 -> ReLU -> 512)."""
+    rng = np.random.Generator(np.random.Philox(600 + m))
+    dims = [4096, 2048, 1024, 512]
+    ws = [(rng.standard_normal((dims[i + 1], dims[i])) * 0.02).astype(np.float32) for i in range(3)]
+    bs = [rng.standard_normal(dims[i + 1]).astype(np.float32) for i in range(3)]
+    x = rng.standard_normal((m, dims[0]), dtype=np.float32)
+    model = Sequential(mode=PER_CHANNEL).input([dims[0]])
+    model.linear(dims[1], ws[0], bs[0]).relu().linear(dims[2], ws[1], bs[1]).relu().linear(dims[3], ws[2], bs[2])
+    for _ in range(2):                                   # second pass: cached weights, same route
+        got = model.forward(x, no_grad=True)
+        cur = x
+        for i in range(3):
+            cur = _oracle_linear(cur, ws[i], bs[i], PER_CHANNEL, relu=i < 2)
+        assert np.array_equal(got, cur)
+    model.release()
+
+
 def test_sequential_builder_rules(hip):
     with pytest.raises(ValueError):
         Sequential().linear(4)                       # no input layer yet

@@ -10,6 +10,7 @@
 // (here: vtl::HipError), never an abort, and there is no CPU fallback in here.
 #pragma once
 
+#include <algorithm>
 #include <cstdint>
 #include <cstdlib>
 #include <cstring>
@@ -531,7 +532,8 @@ public:
         return std::move(pending);
     }
     // `mlp_forward_i8(x, weights, biases, relu_after, slots)`: the whole chain on the device,
-    // int8 codes handed from layer to layer, f32 rows of the last layer back to the host.
+    // int8 codes handed from layer to layer (f32 rows for up to 32 tokens), f32 rows of the
+    // last layer back to the host.
     // An inference call: the parameters count as frozen.
     std::vector<float> mlp_forward_i8(const std::vector<float> &x, int m,
                                       const std::vector<const std::vector<float> *> &weights,
@@ -544,6 +546,28 @@ public:
         if (nl == 0 || biases.size() != nl || relu_after.size() != nl || dims.size() != nl + 1)
             throw std::invalid_argument("mlp_forward_i8: one bias and ReLU flag per weight matrix expected");
         auto x_dev = HipTensor<float>::from_host(x, {m, dims[0]});
+        if (m <= 32) {
+            // A few tokens: every layer quantizes its input inside its own launch (one launch a
+            // layer), so the activations stay f32 between the layers.  Same bits as below.
+            // (Buffers are sized and kept until the end: freeing one waits for the device.)
+            int widest = dims[0];
+            for (size_t i = 1; i < nl; i++)
+                widest = std::max(widest, dims[i]);
+            const HipStorage<uint8_t> &ws = ensure_workspace(m, widest);
+            std::vector<HipTensor<float>> acts;
+            acts.push_back(std::move(x_dev));
+            for (size_t i = 0; i < nl; i++) {
+                QuantizedWeights &q = quantized(weights[i], *weights[i], dims[i + 1], dims[i], *biases[i], true);
+                HipTensor<float> y({m, dims[i + 1]});
+                hip_check(vtl_hip_linear_f32_dynquant((const float *)acts.back().data.ptr,
+                                                      (const int8_t *)q.w_q.data.ptr, (const float *)q.sw.data.ptr,
+                                                      (const float *)q.bias.ptr, (float *)y.data.ptr, m, dims[i + 1],
+                                                      dims[i], relu_after[i] ? 1 : 0, ws.ptr, ws.size),
+                          "vtl_hip_linear_f32_dynquant");
+                acts.push_back(std::move(y));
+            }
+            return acts.back().cpu();
+        }
         auto cur = quantize_i8(x_dev, 0);
         x_dev.release();
         for (size_t i = 0; i + 1 < nl; i++) {

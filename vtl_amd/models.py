@@ -4,7 +4,8 @@ mirror of nn/models/sequential.v:52-220 for input / linear / relu / forward.
 `linear(n)` takes its input width from the previous layer
 (nn/models/sequential_info.v:53-60); `forward` loops over the layers
 (sequential.v:204-215).  Between Linear layers the activations stay on the
-device, as per-token int8 codes when the next layer is a Linear again, and ReLU
+device, as per-token int8 codes when the next layer is a Linear again (as f32
+rows for up to FEW_TOKENS rows), and ReLU
 is folded into the producing Linear's epilogue, in the spirit
 of the reference's GPU activation chain
 (autograd_cuda/device_session_gpu_d_cuda.v:88-181).
@@ -16,6 +17,10 @@ import numpy as np
 from .layers import PER_CHANNEL, HipSession, QuantLinearLayer, kaiming_normal
 from .storage import HipParams
 from .tensor import HipTensor, linear_i8_hip, linear_i8_requant_hip
+
+
+# Rows up to which the library's linear on f32 rows quantizes them inside its own launch.
+FEW_TOKENS = 32
 
 
 class Sequential:
@@ -68,7 +73,12 @@ class Sequential:
                     layer = self.layers[i][1]
                     fuse = i + 1 < n and self.layers[i + 1][0] == "relu"
                     j = i + (2 if fuse else 1)
-                    feeds_linear = self.mode == PER_CHANNEL and j < n and self.layers[j][0] == "linear"
+                    # Up to FEW_TOKENS rows every layer quantizes its input inside its own launch
+                    # (one launch a layer; 1 token through 4096 -> 11008 -> 4096 -> 1024: 23.4
+                    # against 28.0 us), so the activations stay f32 between the layers; with more
+                    # rows the codes go from layer to layer.  The bits are the same either way.
+                    feeds_linear = (self.mode == PER_CHANNEL and j < n and self.layers[j][0] == "linear"
+                                    and x.shape[0] > FEW_TOKENS)
                     if cur_q is None and not feeds_linear:
                         nxt = layer.forward_device(cur, relu=fuse, session=self.session, no_grad=no_grad)
                         cur.release()
