@@ -72,6 +72,8 @@ SHAPES = [(1, 1), (1, 3), (7, 64), (5, 256), (3, 1000), (16, 784), (4, 4096), (2
           (5000, 1000), (70000, 8), (1025, 4092), (3000, 2052), (2, 4092),
           # one row length per workgroup size of the fused kernel
           (9, 512), (10, 2048), (6, 8192), (3, 5000), (5, 11008),
+          # a few very long rows: cut into pieces that meet in an atomic max (and just outside that form)
+          (3, 131072), (5, 262148), (128, 131072), (129, 131072), (2, 131073), (7, 131068),
           # row lengths that are no multiple of four: rows start at any alignment
           (1000, 1001), (300, 4095), (5, 16383), (2, 70001), (4096, 5), (4096, 3), (77, 66), (33, 4099)]
 

@@ -87,6 +87,37 @@ __global__ __launch_bounds__(T) void absmax_rows_kernel(const float *__restrict_
         out[row] = m;
 }
 
+// A few very long rows (16-byte aligned, a multiple of four long): a row is cut into pieces of
+// piece_vecs 16-byte vectors, one workgroup each (block = row * pieces + piece), which meet in
+// an atomic max on out_bits[row] (cleared before).  One workgroup per row, as above, leaves
+// most of the chip idle there: 16 rows of 2^20 took 98 us.
+template <int T>
+__global__ __launch_bounds__(T) void absmax_rows_split_kernel(const float *__restrict__ x, int64_t cols,
+                                                              unsigned pieces, int64_t piece_vecs,
+                                                              unsigned *__restrict__ out_bits)
+{
+    __shared__ float smem[T / 64];
+    const int64_t row = blockIdx.x / pieces;
+    const int64_t piece = blockIdx.x % pieces;
+    const float4_t *xv = reinterpret_cast<const float4_t *>(x + row * cols);
+    const int64_t nv = cols >> 2;
+    const int64_t end = (piece + 1) * piece_vecs < nv ? (piece + 1) * piece_vecs : nv;
+    float m = 0.0f;
+    int64_t i = piece * piece_vecs + threadIdx.x;
+    for (; i + 3 * T < end; i += 4 * T) {
+        const float4_t v0 = __builtin_nontemporal_load(xv + i);
+        const float4_t v1 = __builtin_nontemporal_load(xv + i + T);
+        const float4_t v2 = __builtin_nontemporal_load(xv + i + 2 * T);
+        const float4_t v3 = __builtin_nontemporal_load(xv + i + 3 * T);
+        m = absmax4(absmax4(absmax4(absmax4(m, v0), v1), v2), v3);
+    }
+    for (; i < end; i += T)
+        m = absmax4(m, xv[i]);
+    m = block_max<T>(m, smem);
+    if (threadIdx.x == 0)
+        atomicMax(out_bits + row, __float_as_uint(m));
+}
+
 // Whole-tensor absmax: grid-stride pass, one atomic max per workgroup on the
 // bit pattern (non-negative floats order like unsigned integers).
 // KEEP: ordinary loads, for a tensor that a second pass reads again while the last-level cache
@@ -625,6 +656,37 @@ int launch_absmax_flat(const float *x, int64_t n, unsigned *cell, hipStream_t s)
     return check_launch("absmax_flat_kernel");
 }
 
+int launch_fill_zero(float *p, int64_t n, hipStream_t st);
+
+// Rows so few and so long that one workgroup per row leaves most compute units idle (measured:
+// from 131072 columns on with up to 128 rows, the forms that cut a row into pieces win; 16 rows
+// of 2^20: absmax 98 -> 12 us, quantize 211 -> 36 us).
+inline bool few_long_rows(const float *x, int64_t rows, int64_t cols)
+{
+    return rows <= 128 && cols >= 131072 && cols % 4 == 0 && aligned(x, 16);
+}
+
+// Per-row absmax of such rows into out[rows]: clear, then the pieces' atomic maxima.
+int launch_absmax_rows_split(const float *x, int64_t rows, int64_t cols, float *out, hipStream_t s)
+{
+    int st = launch_fill_zero(out, rows, s);
+    if (st != VTL_HIP_OK)
+        return st;
+    // About 512 workgroups of 1024 threads in all (two per compute unit), a piece a multiple of
+    // what a workgroup loads per step: the rows' maxima share a cache line or two, on which the
+    // atomic maxima queue up (2048 workgroups of 256 threads: 32 us for 64 MiB, this: 12 us).
+    constexpr int T = 1024;
+    const int64_t step = 4 * T;
+    const int64_t share = (rows * (cols >> 2) + 511) / 512;
+    const int64_t piece_vecs = (share + step - 1) / step * step;
+    const int64_t pieces = ((cols >> 2) + piece_vecs - 1) / piece_vecs;
+    if (pieces * rows > kMaxGridX)
+        return VTL_HIP_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL((absmax_rows_split_kernel<T>), dim3((unsigned)(pieces * rows)), dim3(T), 0, s, x, cols,
+                       (unsigned)pieces, piece_vecs, reinterpret_cast<unsigned *>(out));
+    return check_launch("absmax_rows_split_kernel");
+}
+
 int launch_fill_zero(float *p, int64_t n, hipStream_t st)
 {
     const int64_t blocks = (n + 255) / 256;
@@ -724,6 +786,8 @@ int vtl_hip_absmax_f32(const float *x, int64_t rows, int64_t cols, int per_row, 
             return VTL_HIP_OK;
         if (cols == 0)
             return launch_fill_zero(absmax_out, rows, s);
+        if (few_long_rows(x, rows, cols))
+            return launch_absmax_rows_split(x, rows, cols, absmax_out, s);
         const bool vec = aligned(x, 16);  // any row length: the kernel peels to the next 16-byte boundary
         if (vec && cols >= 8192)
             hipLaunchKernelGGL((absmax_rows_kernel<512, 4>), dim3((unsigned)rows), dim3(512), 0, s, x,
@@ -816,6 +880,18 @@ int vtl_hip_quantize_f32_i8(const float *x, int64_t rows, int64_t cols, int per_
     if (!scale_out)
         return VTL_HIP_ERR_INVALID_ARG;
     hipStream_t s = current_stream();
+    if (per_row && few_long_rows(x, rows, cols) && aligned(q, 4)) {
+        // a few very long rows: absmax by pieces, scales in place, then the chunked quantize pass
+        st = launch_absmax_rows_split(x, rows, cols, scale_out, s);
+        if (st != VTL_HIP_OK)
+            return st;
+        hipLaunchKernelGGL(scale_from_absmax_kernel, dim3((unsigned)((rows + 63) / 64)), dim3(64), 0, s, scale_out,
+                           rows);
+        st = check_launch("scale_from_absmax_kernel");
+        if (st != VTL_HIP_OK)
+            return st;
+        return vtl_hip_quantize_with_scale_f32_i8(x, scale_out, rows, cols, 1, q);
+    }
     if (per_row)
         return launch_quantize_rows(x, rows, cols, q, scale_out, s);
     // a small tensor is one "row" of the fused kernel: a single workgroup holds it
