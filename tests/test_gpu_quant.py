@@ -72,6 +72,8 @@ SHAPES = [(1, 1), (1, 3), (7, 64), (5, 256), (3, 1000), (16, 784), (4, 4096), (2
           (5000, 1000), (70000, 8), (1025, 4092), (3000, 2052), (2, 4092),
           # one row length per workgroup size of the fused kernel
           (9, 512), (10, 2048), (6, 8192), (3, 5000), (5, 11008),
+          # many short rows: 16 or 32 lanes a row, several rows per wave (and just outside that form)
+          (4096, 16), (5000, 64), (4097, 100), (4100, 4), (6001, 68), (4096, 128), (4095, 64), (4096, 132), (4099, 256), (5000, 200), (4096, 260),
           # a few very long rows: cut into pieces that meet in an atomic max (and just outside that form)
           (3, 131072), (5, 262148), (128, 131072), (129, 131072), (2, 131073), (7, 131068),
           # row lengths that are no multiple of four: rows start at any alignment

@@ -35,6 +35,23 @@ __device__ __forceinline__ float wave_max(float v)
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
+// Max over each group of SEG = 16, 32 or 64 consecutive lanes (a DPP row, two, or the wave),
+// returned to every lane of the group.
+template <int SEG>
+__device__ __forceinline__ float segment_max(float v)
+{
+    static_assert(SEG == 16 || SEG == 32 || SEG == 64, "a DPP row, two, or the wave");
+    if constexpr (SEG == 64)
+        return wave_max(v);
+    v = dpp_max_step<0xB1, 0xF>(v);
+    v = dpp_max_step<0x4E, 0xF>(v);
+    v = dpp_max_step<0x141, 0xF>(v);
+    v = dpp_max_step<0x140, 0xF>(v);
+    if constexpr (SEG == 32)
+        v = fmaxf(v, __shfl_xor(v, 16));
+    return v;
+}
+
 // Max over the workgroup; every thread gets the result.  smem holds T/64
 // floats and is used once per kernel.
 template <int T>
