@@ -2345,16 +2345,28 @@ int vtl_hip_linear_i8_requant(const int8_t *A, const float *sa, int sa_per_row, 
         !(Y && (size_t)M * (size_t)N * sizeof(int32_t) > ((size_t)256 << 20)) &&
         !tuning().no_fused_requant) {
         // tile kernel leaves int32 sums, one row kernel does epilogue + quantization
-        g.requant_codes = Yq;
-        g.requant_scales = sy;
         int idx, splits;
         choose_config(M, N, K, idx, splits, true);
         const Tuning &tn = tuning();
-        if (tn.gemm_config >= 0 && tn.gemm_config < kNumTileConfigs) {   // VTL_HIP_GEMM_CONFIG, as in launch_gemm
+        const bool config_set = tn.gemm_config >= 0 && tn.gemm_config < kNumTileConfigs;
+        if (config_set) {   // VTL_HIP_GEMM_CONFIG, as in launch_gemm
             idx = tn.gemm_config;
             splits = tn.gemm_splits;
         }
-        return launch_config<true>(idx, g, splits, current_stream());
+        // Without a K split and with a large output the two launches below are the faster
+        // pair: the row kernel of this form reads, per output element, the int32 sum and the
+        // column's scale and bias (12 bytes, two thirds of them the same vectors again for
+        // every row), the row quantizer behind the f32 linear 4.  From about 2.6 M outputs on
+        // that outweighs the tile kernel's cheaper store: 4096^3 85 -> 75 us, 1024 x 11008 x
+        // 4096 64 -> 59 us, 384 x 11008 x 4096 36.0 -> 33.3 us, 256 x 11008 x 4096 23.2 -> 22.4
+        // us; below, this form is 2 to 5 % ahead (256 x 6144 x 4096: 16.0 against 16.9 us).
+        const bool separate_faster = splits == 1 && !config_set && tn.requant_wide <= 0 &&
+                                     (int64_t)M * N >= ((int64_t)5 << 19);
+        if (!separate_faster) {
+            g.requant_codes = Yq;
+            g.requant_scales = sy;
+            return launch_config<true>(idx, g, splits, current_stream());
+        }
     }
     // any other shape: the f32 rows (in the library's staging buffer when the caller wants none),
     // then the row quantizer
