@@ -205,8 +205,13 @@ def test_library_scratch_recorded_into_a_graph_survives_growth_and_never_grows_u
     WB = HipTensor.from_host(rng.integers(-127, 128, (64, kb), dtype=np.int8))
     YB = HipTensor.empty([mb, 64], np.float32)
     capi.call("vtl_hip_memset", XB.ptr, 0, mb * kb * 4)
-    mc = 40960                                      # 160 MiB of codes: asked for under capture only
-    XC, YC = HipTensor.empty([mc, kb], np.float32), HipTensor.empty([mc, 64], np.float32)
+    # Asked for under capture only: 64 GiB of codes, more than the staging buffer can have grown to
+    # whatever ran before in this process (other tests stage f32 rows of outputs beyond 2^32
+    # elements there).  The call must be refused before anything is recorded, so it is handed
+    # the buffers of the eager call; were it accepted, its kernels would only be recorded into
+    # a graph that is destroyed without a launch.
+    mc = 1 << 24
+    XC, YC = XB, YB
 
     def small():
         capi.call("vtl_hip_linear_f32_dynquant", X.ptr, W.ptr, SW.ptr, None, Y.ptr, m, n, k, 0, None, 0)
@@ -227,7 +232,7 @@ def test_library_scratch_recorded_into_a_graph_survives_growth_and_never_grows_u
             assert hiprt.hipGraphLaunch(gexec, stream) == 0
             capi.call("vtl_hip_sync")
             assert np.array_equal(Y.cpu(), oracle.linear_f32_dynquant(xr, w, sw, None)), f"replay {rep}"
-        # under capture the buffer may be used, never grown: 160 MiB of codes do not fit what exists
+        # under capture the buffer may be used, never grown: 64 GiB of codes do not fit what exists
         assert hiprt.hipStreamBeginCapture(stream, 0) == 0
         st = capi.status("vtl_hip_linear_f32_dynquant", XC.ptr, WB.ptr, SW.ptr, None, YC.ptr, mc, 64, kb, 0, None, 0)
         graph2 = C.c_void_p()
@@ -242,7 +247,7 @@ def test_library_scratch_recorded_into_a_graph_survives_growth_and_never_grows_u
         if graph:
             hiprt.hipGraphDestroy(graph)
         hiprt.hipStreamDestroy(stream)
-        for t in (X, W, SW, Y, XB, WB, YB, XC, YC):
+        for t in (X, W, SW, Y, XB, WB, YB):
             t.release()
 
 

@@ -2049,10 +2049,10 @@ int launch_skinny(const GemmArgs &g, int nwave, hipStream_t st)
 // launch of 6.1 us where the tile kernels need a K split and a second launch to fill the chip
 // (10.0 us); 33x4096x2048 4.9 against 8.1 us, 256x1024x11008 10.9 against 13.7 us.  Returns
 // the number of waves per workgroup (4: at most one round of workgroups, one per compute unit;
-// 2: up to two rounds of two per compute unit), or 0 where the tile kernels are as fast or
+// the tuning knob can ask for 2 or 8), or 0 where the tile kernels are as fast or
 // faster (short K: everything is launch-bound; more blocks: the tiles' operand reuse wins;
 // few blocks with a very long K: the tile kernels' finer K split wins).  Measured over
-// K = 256 ... 8192 and 4 ... 512 blocks.
+// K = 256 ... 8192 and 4 ... 1024 blocks.
 inline int skinny_blocks_waves(int M, int N, int K)
 {
     if (tuning().skinny_tiled >= 0)   // 1 / 0 force the choice (tests, tuning)
@@ -2060,10 +2060,13 @@ inline int skinny_blocks_waves(int M, int N, int K)
     const int64_t blocks = (int64_t)((M + 31) / 32) * ((N + 31) / 32);
     if (K < 1024)
         return 0;
+    // Timed again with the two routes alternating (after an idle gap the first timing of a launch
+    // this short reads several percent high): up to 256 blocks 0.61 to 0.86 of the tile kernels'
+    // time for K <= 4096 and 0.61 to 0.93 at K = 8192 from 64 blocks on (level below that); with
+    // 257 to 512 blocks, two waves each, 8 to 12 % behind at K = 1024, 0 to 9 % behind at K = 2048
+    // and level at K = 4096, so that range went back to the tile kernels.
     if (blocks <= 256)
-        return (K <= 4096 || blocks >= 96) ? 4 : 0;
-    if (blocks <= 512)
-        return K <= 4096 ? 2 : 0;
+        return (K <= 4096 || blocks >= 64) ? 4 : 0;
     return 0;
 }
 
@@ -2166,17 +2169,24 @@ inline bool gemv_rows_applies(const void *rows, const void *w, int M, int N, int
 // Where the few-token kernel beats the MFMA weight-streaming kernel (measured, N = 64 ... 28672,
 // K = 256 ... 8192): its dot4 work grows with M * N * K while the other's does not, but it has no
 // LDS staging and a lower fixed cost.  Shapes the other kernel cannot take (K % 256 != 0) come here.
-inline bool gemv_rows_faster(int M, int N, int K)
+// `against_staged_launch`: the narrower rule by which the f32 entry decides between quantizer +
+// this kernel and the weight-streaming launch that quantizes the rows itself (its sweep was made
+// with that rule; the one launch keeps shapes there that this kernel wins as a plain linear).
+inline bool gemv_rows_faster(int M, int N, int K, bool against_staged_launch = false)
 {
     if (tuning().gemv_rows >= 0)   // 1 / 0 force the choice (tests, tuning)
         return tuning().gemv_rows != 0;
     if (M <= 2 || K % 256 != 0 || N < 2048)   // few weight rows: never slower, 1.8x faster from K = 4096 on
         return true;
+    if (against_staged_launch)
+        return M <= 4 ? (K >= 2048 || N <= 8192) : (int64_t)N * K <= ((int64_t)4 << 20);
+    // As a plain int8 linear, timed with the two kernels alternating (N = 512 ... 14336, K = 1024
+    // ... 8192, cached / from HBM): 3 and 4 rows 0.72 to 0.93 of the other kernel's time up to
+    // 8192 x 4096 and level beyond; 5 to 8 rows 0.80 to 0.94 / 0.89 to 1.0 up to N * K = 8 M
+    // (6 x 2048 x 4096: 4.7 against 5.9 us), level at 16 M, and 1.1 to 1.25 from 14336 x 1024 on.
     if (M <= 4)
-        return K >= 2048 || N <= 8192;
-    // 5 to 8 rows: only small products (against four waves of the other kernel, which these
-    // shapes get: 8 x 4096 x 4096 5.5 against 4.8 us)
-    return (int64_t)N * K <= ((int64_t)4 << 20);
+        return true;
+    return (int64_t)N * K <= ((int64_t)8 << 20);
 }
 
 // Quantizing the rows inside every workgroup of the few-token kernel costs about 15 instructions
@@ -2202,7 +2212,9 @@ inline bool gemv_applies(const void *row, const void *w, int N, int K)
 // which the tile kernels could only fill the chip with by cutting K (a second launch).
 inline bool small_product_faster(int64_t t32, int K)
 {
-    return t32 <= 64 && K <= 2048;
+    // (up to 128 tiles below K = 1024, where the 32 x 32-block route does not go: 256 x 512 x 512
+    // 3.8 against 4.5 us on the tile kernels)
+    return (t32 <= 64 && K <= 2048) || (t32 <= 128 && K < 1024);
 }
 inline int small_product_waves(int64_t t32, int K)
 {
@@ -2440,7 +2452,7 @@ int vtl_hip_linear_f32_dynquant(const float *X, const int8_t *Wq, const float *s
         GemmArgs g{nullptr, Wq, Y, nullptr, sw, bias, M, N, K, 1, 1, relu ? 1 : 0, 1, nullptr, X, 0};
         return launch_gemv_rows<true, true>(g, current_stream());
     }
-    const bool staged = stage_inside_launch_faster(M, N, K, gemv_rows_applies(X, Wq, M, N, K) && gemv_rows_faster(M, N, K)) &&
+    const bool staged = stage_inside_launch_faster(M, N, K, gemv_rows_applies(X, Wq, M, N, K) && gemv_rows_faster(M, N, K, true)) &&
                         aligned16(X) && aligned16(Wq) && tuning().gemm_config < 0 && !tuning().no_fused_decode;
     if (!workspace) {   // no caller scratch: stage in the library's own buffer
         workspace = vtlhip::library_workspace(vtl_hip_linear_f32_dynquant_workspace(M, K), 1);
