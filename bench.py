@@ -563,6 +563,31 @@ def _bench_chain(timed, out):
         "weights_from_hbm": {"us": us_hbm, "TOPS": ops / us_hbm / 1e6, "weight_GB/s": wbytes / us_hbm / 1e3,
                              "note": "6 copies of the three matrices in turn (564 MB)"},
         "per_layer (input quantize + linear/ReLU/requantize, same, linear to f32)": layers}
+    # The same three layers with a few tokens: the layers hand f32 rows on and each quantizes its
+    # input inside its own launch (what Sequential.forward and mlp_forward_i8 do up to 32 rows).
+    few = {}
+    for mt in (1, 8, 32):
+        Xs = HipTensor.from_host(x_host[:mt])
+        Hs = [HipTensor.empty([mt, dims[i + 1]], np.float32) for i in range(3)]
+        need = int(capi.lib().vtl_hip_linear_f32_dynquant_workspace(mt, max(dims[:3])))
+        Wk = HipTensor.empty([need], np.uint8)
+
+        def few_chain(ws_=None, mt=mt, Xs=Xs, Hs=Hs, Wk=Wk):
+            ws_ = Ws if ws_ is None else ws_
+            src = Xs
+            for i in range(3):
+                capi.call("vtl_hip_linear_f32_dynquant", src.ptr, ws_[i].ptr, Ss[i].ptr, None, Hs[i].ptr, mt,
+                          dims[i + 1], dims[i], 1 if i < 2 else 0, Wk.ptr, Wk.size)
+                src = Hs[i]
+
+        def few_streaming(few_chain=few_chain):
+            few_chain(sets[turn[0] % len(sets)])
+            turn[0] += 1
+        few[f"M={mt}"] = {"us": timed(few_chain), "weights_from_hbm_us": timed(few_streaming)}
+        capi.call("vtl_hip_sync")
+        for h in [Xs, Wk] + Hs:
+            h.release()
+    out["configs[4] int8 MLP chain 256x4096->11008->4096->1024"]["few_tokens (f32 rows from layer to layer, one launch a layer)"] = few
     capi.call("vtl_hip_sync")
     for h in Ss + Qs + Sx + [X, Y] + [w for st in sets for w in st]:
         h.release()
