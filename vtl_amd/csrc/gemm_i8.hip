@@ -65,6 +65,9 @@ struct GemmArgs {
     int sync_slot;
     int spin_limit;
     unsigned stage_target;
+    // Weight-streaming kernel with up to 32 rows (every weight is read once): read the weights
+    // with non-temporal loads.  Set by the size of the matrix, see stream_weights_from.
+    int stream_weights;
 };
 
 // LDS tiles are rows of BK bytes (BK/16 chunks of 16 bytes).  The chunk index
@@ -978,9 +981,16 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_skinny_kernel(const GemmArg
     auto issue_w = [&](int c, int st) {
         char *sw_ = ring + st * SLOT;
         const int64_t ko = (int64_t)c * BK;
+        // (the cache policy is part of the instruction: one copy of the loads for each)
+        if (g.stream_weights) {
 #pragma unroll
-        for (int j = 0; j < WLOADS; j++)
-            __builtin_amdgcn_global_load_lds(VTL_GPTR(pw[j] + ko), VTL_LPTR(sw_ + j * 1024), 16, 0, 0);
+            for (int j = 0; j < WLOADS; j++)
+                __builtin_amdgcn_global_load_lds(VTL_GPTR(pw[j] + ko), VTL_LPTR(sw_ + j * 1024), 16, 0, 2);
+        } else {
+#pragma unroll
+            for (int j = 0; j < WLOADS; j++)
+                __builtin_amdgcn_global_load_lds(VTL_GPTR(pw[j] + ko), VTL_LPTR(sw_ + j * 1024), 16, 0, 0);
+        }
     };
     auto issue_x = [&](int c, int st) {
         char *sx_ = ring + st * SLOT + WCHUNK;
@@ -1202,7 +1212,7 @@ __device__ __forceinline__ int wave_sum_i32(int v)
 // cache, non-temporal ones measured 20-40 % slower), two rows are in flight
 // while the current one goes through 4 * KV dot4 instructions and a
 // cross-lane sum.  Requires K % 16 == 0, the row and Wq 16-byte aligned.
-template <int KV, int NWAVE, bool DYNQ, bool F32OUT>
+template <int KV, int NWAVE, bool DYNQ, bool F32OUT, bool WNT = false>
 __global__ __launch_bounds__(64 * NWAVE) void linear_gemv_kernel(const GemmArgs g)
 {
     constexpr int T = 64 * NWAVE;
@@ -1233,7 +1243,7 @@ __global__ __launch_bounds__(64 * NWAVE) void linear_gemv_kernel(const GemmArgs 
         const v4i *p = reinterpret_cast<const v4i *>(g.Bt + r * K) + lane;
 #pragma unroll
         for (int j = 0; j < KV; j++)
-            dst[j] = (64 * j + lane < kv) ? p[64 * j] : v4i{0, 0, 0, 0};
+            dst[j] = (64 * j + lane < kv) ? (WNT ? __builtin_nontemporal_load(p + 64 * j) : p[64 * j]) : v4i{0, 0, 0, 0};
     };
 #pragma unroll
     for (int d = 0; d < DEPTH; d++)
@@ -1926,9 +1936,23 @@ inline int skinny_waves_few_rows(int N, int K)
     return ((N <= 8192 && K >= 2048) || K >= 8192) ? 4 : 2;
 }
 
+// Whether a decode kernel reads an N x K weight matrix with non-temporal loads: from `mib` MiB
+// on.  A model made of such matrices does not stay in the 256 MB last-level cache from one
+// step to the next, and streaming from HBM the loads are worth 2 to 8 % (N = 14336, K = 4096:
+// 1 row 11.7 -> 11.1 us, 8 rows 14.4 -> 13.7 us, 32 rows 16.6 -> 16.1 us).  The price is paid by
+// a caller who repeats the launch on one matrix that would have stayed in that cache: nothing
+// for the single-row kernel (it gains there too, 10.1 -> 9.2 us), but 12 to 23 % for the
+// weight-streaming kernel on matrices of 32 to 45 MiB and 0 to 12 % on larger ones, which is
+// why it starts at 48 MiB and the single-row kernel at 8 (below, it is level or 5 % behind).
+// The few-token kernel (2 to 8 rows) keeps ordinary loads: 3 to 6 % behind from HBM, up to 12 %
+// ahead on a repeated matrix.
+inline bool stream_weights_from(int N, int K, int mib) { return (int64_t)N * K >= ((int64_t)mib << 20); }
+
 template <int NWAVE, int STAGES, int XJ, bool F32OUT, bool STAGEQ = false>
-int launch_skinny_cfg(const GemmArgs &g, hipStream_t st)
+int launch_skinny_cfg(const GemmArgs &g_in, hipStream_t st)
 {
+    GemmArgs g = g_in;
+    g.stream_weights = (g.M <= 32 && stream_weights_from(g.N, g.K, 48)) ? 1 : 0;   // (one block of rows: every weight is read once)
     constexpr int lds = NWAVE * STAGES * (8192 + XJ * 2048);
     static_assert(lds >= NWAVE * 4096, "room for the partial tiles");
     static PerDevice<DoneFlag> done_flag;
@@ -2077,8 +2101,9 @@ inline int gemv_max_waves(int K) { return K <= 6144 ? 4096 : 2048; }
 
 // Single-token linear (M = 1, K % 16 == 0, K <= 14336, operands 16-byte aligned).
 template <bool DYNQ, bool F32OUT>
-int launch_gemv(const GemmArgs &g, hipStream_t st)
+int launch_gemv(const GemmArgs &g_in, hipStream_t st)
 {
+    const GemmArgs &g = g_in;
     constexpr int NWAVE = 8;
     // every wave the same number of rows
     const int max_waves = gemv_max_waves(g.K);
@@ -2087,20 +2112,29 @@ int launch_gemv(const GemmArgs &g, hipStream_t st)
         return VTL_HIP_ERR_UNSUPPORTED;
     const int64_t waves = (g.N + rows_per_wave - 1) / rows_per_wave;
     const dim3 grid((unsigned)((waves + NWAVE - 1) / NWAVE)), block(64 * NWAVE);
+    const bool wnt = stream_weights_from(g.N, g.K, 8);   // the cache policy is part of the load instruction
+#define VTL_GEMV(KV)                                                                                        \
+    do {                                                                                                    \
+        if (wnt)                                                                                            \
+            hipLaunchKernelGGL((linear_gemv_kernel<KV, NWAVE, DYNQ, F32OUT, true>), grid, block, 0, st, g); \
+        else                                                                                                \
+            hipLaunchKernelGGL((linear_gemv_kernel<KV, NWAVE, DYNQ, F32OUT, false>), grid, block, 0, st, g); \
+    } while (0)
     switch ((g.K + 1023) / 1024) {
-    case 1: hipLaunchKernelGGL((linear_gemv_kernel<1, NWAVE, DYNQ, F32OUT>), grid, block, 0, st, g); break;
-    case 2: hipLaunchKernelGGL((linear_gemv_kernel<2, NWAVE, DYNQ, F32OUT>), grid, block, 0, st, g); break;
-    case 3: hipLaunchKernelGGL((linear_gemv_kernel<3, NWAVE, DYNQ, F32OUT>), grid, block, 0, st, g); break;
-    case 4: hipLaunchKernelGGL((linear_gemv_kernel<4, NWAVE, DYNQ, F32OUT>), grid, block, 0, st, g); break;
+    case 1: VTL_GEMV(1); break;
+    case 2: VTL_GEMV(2); break;
+    case 3: VTL_GEMV(3); break;
+    case 4: VTL_GEMV(4); break;
     case 5:
-    case 6: hipLaunchKernelGGL((linear_gemv_kernel<6, NWAVE, DYNQ, F32OUT>), grid, block, 0, st, g); break;
+    case 6: VTL_GEMV(6); break;
     case 7:
-    case 8: hipLaunchKernelGGL((linear_gemv_kernel<8, NWAVE, DYNQ, F32OUT>), grid, block, 0, st, g); break;
+    case 8: VTL_GEMV(8); break;
     case 9:
     case 10:
-    case 11: hipLaunchKernelGGL((linear_gemv_kernel<11, NWAVE, DYNQ, F32OUT>), grid, block, 0, st, g); break;
-    default: hipLaunchKernelGGL((linear_gemv_kernel<14, NWAVE, DYNQ, F32OUT>), grid, block, 0, st, g); break;
+    case 11: VTL_GEMV(11); break;
+    default: VTL_GEMV(14); break;
     }
+#undef VTL_GEMV
     return check_launch("linear_gemv_kernel");
 }
 
