@@ -1391,7 +1391,7 @@ __device__ __forceinline__ int wave_sum_rows(int (&a)[MR], int lane)
 // 64 / MR weight rows at a time (lane l: row l % MR, weight row l / MR of the
 // batch) and then scaled and stored.  Requires K % 16 == 0, K <= 1024 * KV,
 // operands 16-byte aligned.
-template <int KV, int MR, int DEPTH, bool DYNQ, bool F32OUT>
+template <int KV, int MR, int DEPTH, bool DYNQ, bool F32OUT, bool WNT = false>
 __global__ __launch_bounds__(512) void linear_gemv_rows_kernel(const GemmArgs g)
 {
     constexpr int NWAVE = 8;
@@ -1428,7 +1428,7 @@ __global__ __launch_bounds__(512) void linear_gemv_rows_kernel(const GemmArgs g)
         const v4i *p = reinterpret_cast<const v4i *>(g.Bt + r * K) + lane;
 #pragma unroll
         for (int j = 0; j < KV; j++)
-            dst[j] = (64 * j + lane < kv) ? p[64 * j] : v4i{0, 0, 0, 0};
+            dst[j] = (64 * j + lane < kv) ? (WNT ? __builtin_nontemporal_load(p + 64 * j) : p[64 * j]) : v4i{0, 0, 0, 0};
     };
 #pragma unroll
     for (int d = 0; d < DEPTH; d++)
@@ -1943,9 +1943,9 @@ inline int skinny_waves_few_rows(int N, int K)
 // a caller who repeats the launch on one matrix that would have stayed in that cache: nothing
 // for the single-row kernel (it gains there too, 10.1 -> 9.2 us), but 12 to 23 % for the
 // weight-streaming kernel on matrices of 32 to 45 MiB and 0 to 12 % on larger ones, which is
-// why it starts at 48 MiB and the single-row kernel at 8 (below, it is level or 5 % behind).
-// The few-token kernel (2 to 8 rows) keeps ordinary loads: 3 to 6 % behind from HBM, up to 12 %
-// ahead on a repeated matrix.
+// why it and the few-token kernel (2 to 8 rows: 3 to 6 % from HBM, 12 % behind on a repeated
+// matrix of 32 to 45 MiB) start at 48 MiB and the single-row kernel at 8 (below, it is level or
+// 5 % behind).
 inline bool stream_weights_from(int N, int K, int mib) { return (int64_t)N * K >= ((int64_t)mib << 20); }
 
 template <int NWAVE, int STAGES, int XJ, bool F32OUT, bool STAGEQ = false>
@@ -2155,7 +2155,10 @@ int launch_gemv_rows_kv(const GemmArgs &g, hipStream_t st)
     if constexpr (DYNQ && MR * KV > 8) {
         return VTL_HIP_ERR_UNSUPPORTED;  // not routed here: a quantizer launch of its own is cheaper
     } else {
-        hipLaunchKernelGGL((linear_gemv_rows_kernel<KV, MR, DEPTH, DYNQ, F32OUT>), grid, block, 0, st, g);
+        if (stream_weights_from(g.N, g.K, 48))   // (the cache policy is part of the load instruction)
+            hipLaunchKernelGGL((linear_gemv_rows_kernel<KV, MR, DEPTH, DYNQ, F32OUT, true>), grid, block, 0, st, g);
+        else
+            hipLaunchKernelGGL((linear_gemv_rows_kernel<KV, MR, DEPTH, DYNQ, F32OUT, false>), grid, block, 0, st, g);
         return check_launch("linear_gemv_rows_kernel");
     }
 }
