@@ -256,7 +256,9 @@ def test_session_reuses_buffers_on_second_forward(hip):
                                  (3, 2048, 1024), (4, 4099, 1040), (4, 2048, 2048), (3, 2051, 272),
                                  (5, 2048, 512), (8, 2050, 1024), (7, 9000, 1008), (6, 2048, 16 * 17),
                                  (8, 70001, 256), (2, 1, 256), (3, 7, 2048), (8, 64, 1024), (4, 100, 272),
-                                 (2, 1536, 4096)])
+                                 (2, 1536, 4096),
+                                 # 48 MiB of weights and more: the instances with non-temporal weight loads
+                                 (2, 14336, 4096), (4, 16400, 3072), (2, 8192, 8192), (7, 12300, 4096)])
 def test_few_token_fused_decode_equals_two_launch_path(hip, mnk, knobs):
     """2 to 8 tokens with short rows take the few-token kernel whose workgroups quantize the
     rows themselves (forced here for every size it is built for); it must give the bits of
