@@ -148,6 +148,30 @@ def test_mlp_chain_with_few_tokens(hip, m):
     model.release()
 
 
+@pytest.mark.parametrize("mnk", [(2, 2048, 1024), (4, 4100, 2048), (8, 2050, 1024), (16, 3000, 4096), (32, 2048, 2048)])
+def test_weight_cache_policy_does_not_change_the_bits(hip, mnk, knobs):
+    """The kernels for 2 to 32 rows read large weight matrices with non-temporal loads
+    (VTL_HIP_STREAM_WEIGHTS_MIB sets the size; 0: every matrix): same results either way."""
+    m, n, k = mnk
+    rng = np.random.Generator(np.random.Philox(m + n + k))
+    x = rng.standard_normal((m, k), dtype=np.float32)
+    w = rng.integers(-127, 128, (n, k), dtype=np.int8)
+    sw = (rng.uniform(0.5, 1.5, n) * 1e-3).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    X, W, SW, B = dev(x), dev(w), dev(sw), dev(bias)
+    want = oracle.linear_f32_dynquant(x, w, sw, bias, relu=True, threads=CPU_THREADS)
+    for mib in ("0", "1000000"):
+        knobs.setenv("VTL_HIP_STREAM_WEIGHTS_MIB", mib)
+        for rows_kernel in (None, "1", "0"):
+            if rows_kernel is None:
+                knobs.delenv("VTL_HIP_GEMV_ROWS", raising=False)
+            else:
+                knobs.setenv("VTL_HIP_GEMV_ROWS", rows_kernel)
+            assert np.array_equal(linear_f32_dynquant_hip(X, W, SW, B, relu=True).cpu(), want), (mib, rows_kernel)
+    for h in (X, W, SW, B):
+        h.release()
+
+
 def test_sequential_builder_rules(hip):
     with pytest.raises(ValueError):
         Sequential().linear(4)                       # no input layer yet

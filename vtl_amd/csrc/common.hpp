@@ -75,6 +75,7 @@ struct Tuning {
     bool quant_four_launches = false;  // VTL_HIP_QUANT_FOUR_LAUNCHES: whole-tensor quantize as clear + absmax + scale + quantize (tests)
     bool no_fused_decode = false;   // VTL_HIP_NO_FUSED_DECODE: quantizer launch in front of the linear
     int stage_spin = 4096;          // VTL_HIP_STAGE_SPIN: polls a workgroup of the decode launch waits for the quantized rows (0: none, tests)
+    int stream_weights_mib = 48;    // VTL_HIP_STREAM_WEIGHTS_MIB: weight matrices of this many MiB and more are read with non-temporal loads by the kernels for 2 to 32 rows (0: always)
     int skinny_tiled = -1;          // VTL_HIP_SKINNY_TILED: 1 / 0 force the 32x32-block weight-streaming kernel for M > 32
     int skinny_waves = 4;           // VTL_HIP_SKINNY_WAVES: 2, 4 or 8 waves (K ranges) per workgroup there
     int matmul_tile = 0;            // VTL_HIP_MATMUL_TILE: 128 / 64 force the f64-accumulating tile

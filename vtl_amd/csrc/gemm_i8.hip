@@ -1945,14 +1945,15 @@ inline int skinny_waves_few_rows(int N, int K)
 // weight-streaming kernel on matrices of 32 to 45 MiB and 0 to 12 % on larger ones, which is
 // why it and the few-token kernel (2 to 8 rows: 3 to 6 % from HBM, 12 % behind on a repeated
 // matrix of 32 to 45 MiB) start at 48 MiB and the single-row kernel at 8 (below, it is level or
-// 5 % behind).
+// 5 % behind).  A caller whose model is made of smaller matrices and does not fit that cache
+// lowers the first limit with VTL_HIP_STREAM_WEIGHTS_MIB (16 for 4096 x 4096 and up).
 inline bool stream_weights_from(int N, int K, int mib) { return (int64_t)N * K >= ((int64_t)mib << 20); }
 
 template <int NWAVE, int STAGES, int XJ, bool F32OUT, bool STAGEQ = false>
 int launch_skinny_cfg(const GemmArgs &g_in, hipStream_t st)
 {
     GemmArgs g = g_in;
-    g.stream_weights = (g.M <= 32 && stream_weights_from(g.N, g.K, 48)) ? 1 : 0;   // (one block of rows: every weight is read once)
+    g.stream_weights = (g.M <= 32 && stream_weights_from(g.N, g.K, tuning().stream_weights_mib)) ? 1 : 0;   // (one block of rows: every weight is read once)
     constexpr int lds = NWAVE * STAGES * (8192 + XJ * 2048);
     static_assert(lds >= NWAVE * 4096, "room for the partial tiles");
     static PerDevice<DoneFlag> done_flag;
@@ -2155,7 +2156,7 @@ int launch_gemv_rows_kv(const GemmArgs &g, hipStream_t st)
     if constexpr (DYNQ && MR * KV > 8) {
         return VTL_HIP_ERR_UNSUPPORTED;  // not routed here: a quantizer launch of its own is cheaper
     } else {
-        if (stream_weights_from(g.N, g.K, 48))   // (the cache policy is part of the load instruction)
+        if (stream_weights_from(g.N, g.K, tuning().stream_weights_mib))   // (the cache policy is part of the load instruction)
             hipLaunchKernelGGL((linear_gemv_rows_kernel<KV, MR, DEPTH, DYNQ, F32OUT, true>), grid, block, 0, st, g);
         else
             hipLaunchKernelGGL((linear_gemv_rows_kernel<KV, MR, DEPTH, DYNQ, F32OUT, false>), grid, block, 0, st, g);

@@ -74,6 +74,9 @@ static const Tuning *read_tuning(bool force)
     t->stage_spin = number("VTL_HIP_STAGE_SPIN", 4096);
     if (t->stage_spin < 0 || t->stage_spin > (1 << 20))
         t->stage_spin = 4096;
+    t->stream_weights_mib = number("VTL_HIP_STREAM_WEIGHTS_MIB", 48);
+    if (t->stream_weights_mib < 0 || t->stream_weights_mib > (1 << 20))
+        t->stream_weights_mib = 48;
     t->skinny_tiled = number("VTL_HIP_SKINNY_TILED", -1);
     t->skinny_waves = number("VTL_HIP_SKINNY_WAVES", 4);
     t->matmul_tile = number("VTL_HIP_MATMUL_TILE", 0);
